@@ -75,6 +75,12 @@ typedef struct mfq_amd_projection {
 
 const char* mfq_amd_last_error(void);
 int mfq_amd_abi_version(void);
+/* One-time set-up of the current device: the SwiGLU sigmoid table (the reference builds the same table once per
+ * process with moe_swiglu_sigmoid_table_cuda, mfq/kernels/cuda/moe.cu:2657-2665) and the dynamic-LDS limits of the
+ * kernels that need more than 64 KB.  Allocates and synchronises.  Optional: mfq_amd_moe_ffn_create, and the first
+ * call on a device of mfq_amd_swiglu, of a route plan over more than 1024 pairs or of a prefill-sized projection do
+ * it themselves (thread-safe), so call it beforehand when that first call would sit inside a stream capture. */
+int mfq_amd_init(void);
 
 /* ---------------------------------------------------------------------------
  * Loading: canonical blob -> runtime packed layout.
@@ -187,7 +193,9 @@ typedef struct mfq_amd_moe_ffn_config {
     int32_t x_dtype;           /* MFQ_AMD_F32 / F16 / BF16 */
     int32_t out_dtype;         /* MFQ_AMD_F32 or MFQ_AMD_F16 */
     float swiglu_limit;        /* > 0: clamped variant (mfe_ffn.h:111-114) */
-    int32_t decode_token_limit;/* tokens <= limit use the streaming GEMV kernels, more use the grouped GEMM; 0 = default (32) */
+    int32_t decode_token_limit;/* tokens <= limit use the streaming GEMV kernels, more use the grouped GEMM; 0 = default (32).
+                                * Clamped to 1024 / top_k: a decode plan is one thread per routed pair
+                                * (mfq_amd_moe_ffn_decode_limit gives the value create will use). */
     int32_t launch_mode;       /* decode: 0 = one launch per stage covering every format (blocks sorted by
                                   format), 1 = one launch per format and stage */
     int32_t reserved[3];
@@ -197,6 +205,9 @@ typedef struct mfq_amd_moe_ffn_config {
  * captured into a HIP graph (workspaces are fixed at create, as the reference fixes them per capacity
  * bucket, ops/include/mfe_weight.h:49-72). */
 int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_amd_moe_ffn** out);
+/* The decode token limit create uses for a requested limit (0 = default) and top_k; pure, needs no device.
+ * Counterpart of the capacity buckets the reference fixes per runtime (ops/include/mfe_weight.h:49-72). */
+int32_t mfq_amd_moe_ffn_decode_limit(int32_t requested, int32_t top_k);
 int mfq_amd_moe_ffn_run(mfq_amd_moe_ffn* ffn, const void* x_dev, const int32_t* ids_dev,
                         const float* route_weights_dev, int32_t tokens, void* out_dev, void* stream);
 /* The same layer with routing fused in: softmax top-k of logits_dev[tokens, experts] (arguments as
@@ -233,7 +244,8 @@ int mfq_amd_grouped_matmul(const mfq_amd_moe_tensor* tensor, const void* x_dev, 
                            void* out_f16_dev, void* workspace_dev, int64_t workspace_bytes, void* stream);
 
 /* hidden = swiglu(gate, up) with the reference's fp16 rounding chain
- * (mfq/kernels/cuda/mfe_ffn.h:105-118; cuda/storage/moe_ffn_pipeline.cpp:154-169). */
+ * (mfq/kernels/cuda/mfe_ffn.h:105-118; cuda/storage/moe_ffn_pipeline.cpp:154-169).  Uses the device's sigmoid
+ * table (see mfq_amd_init). */
 int mfq_amd_swiglu(const void* gate_f16_dev, const void* up_f16_dev, int64_t count, float swiglu_limit,
                    void* hidden_f16_dev, void* stream);
 /* out[t, c] = sum_r w[t, r] * pair[t, r, c], fp32, routes ascending.  Replaces

@@ -54,6 +54,8 @@ EXPORTS = {
     # name: (restype, argtypes)
     "mfq_amd_last_error": (C.c_char_p, []),
     "mfq_amd_abi_version": (C.c_int, []),
+    "mfq_amd_init": (C.c_int, []),
+    "mfq_amd_moe_ffn_decode_limit": (C.c_int32, [C.c_int32, C.c_int32]),
     "mfq_amd_tensor_load": (C.c_int, [C.c_char_p, C.c_void_p, C.c_int64, C.c_int32, c_void_pp]),
     "mfq_amd_tensor_host_view": (C.c_int, [C.c_void_p, C.POINTER(Projection)]),
     "mfq_amd_tensor_upload": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.POINTER(Projection)]),

@@ -43,7 +43,14 @@ void validate_projection(const mfq_amd_projection& p, int local_expert) {
         MFQ_REQUIRE(p.groups == 1 + (p.input_width - 1) / p.group_size, "NINT group count does not match width");
         for (int i = 0; i < 7; ++i) MFQ_REQUIRE(p.fields[i] != nullptr, "missing packed NINT storage");
         MFQ_REQUIRE(p.local_experts == 1 || p.q_expert_stride > 0, "MFE NINT pools need q_expert_stride");
-        MFQ_REQUIRE(p.sizes[0] >= (p.local_experts - 1) * p.q_expert_stride, "packed NINT row exceeds storage");
+        MFQ_REQUIRE(p.uniform_bits >= 0 && p.uniform_bits <= 8, "NINT code width must be 1..8 (0 = per-row widths)");
+        // the code stream of one expert: rows * groups * group_size codes of uniform_bits each (per-row widths: at
+        // least one bit each); every expert's stream must fit its stride and the last one the storage
+        const int64_t codes = static_cast<int64_t>(p.output_rows) * p.groups * p.group_size;
+        const int64_t stream = (codes * (p.uniform_bits ? p.uniform_bits : 1) + 7) / 8;
+        MFQ_REQUIRE(p.q_expert_stride >= 0 && (p.local_experts == 1 || p.q_expert_stride >= stream),
+                    "packed NINT expert stream exceeds its stride");
+        MFQ_REQUIRE(p.sizes[0] >= (p.local_experts - 1) * p.q_expert_stride + stream, "packed NINT row exceeds storage");
     } else if (p.family == MFQ_AMD_FAMILY_NVQ) {
         if (!nvq_format_supported(p.format)) fail_unsupported("NVQ runtime format is not implemented");
         MFQ_REQUIRE(p.group_size == 24, "NVQ requires 24-value groups");

@@ -26,8 +26,14 @@ struct Reader {
     const uint8_t* data;
     int64_t size;
     int64_t off = 0;
+    int64_t left() const { return size - off; }
+    // compares against the bytes that remain, so that a length near the top of the range cannot wrap the sum
+    // (cpp_runtime/backends/cuda/ops/moe.cpp:70-87 does the same)
     void need(int64_t n, const char* what) const {
-        if (n < 0 || off + n > size) fail_invalid(std::string("truncated ") + what);
+        if (n < 0 || n > size - off) fail_invalid(std::string("truncated ") + what);
+    }
+    void need_u64(uint64_t n, const char* what) const {
+        if (n > static_cast<uint64_t>(size - off)) fail_invalid(std::string("truncated ") + what);
     }
     template <class T> T get(const char* what) {
         need(sizeof(T), what);
@@ -44,11 +50,18 @@ struct Reader {
     }
 };
 
-inline int64_t stream_bytes(int64_t count, int bits) { return (count * bits + 7) / 8; }
+// a * b for non-negative operands; fails instead of wrapping (every product here counts bytes or bits of a blob)
+inline int64_t checked_mul(int64_t a, int64_t b, const char* what) {
+    if (a < 0 || b < 0 || (b != 0 && a > (int64_t(1) << 59) / b)) fail_invalid(std::string("oversized ") + what);
+    return a * b;
+}
+
+inline int64_t stream_bytes(int64_t count, int bits) { return (checked_mul(count, bits, "bit stream") + 7) / 8; }
 
 // LSB-first bit stream reader for metadata streams (values <= 8 bits).
 std::vector<uint8_t> unpack_bits(Reader& in, int64_t count, int bits, const char* what) {
-    const uint8_t* p = in.take(stream_bytes(count, bits), what);
+    MFQ_REQUIRE(count >= 0 && bits >= 1 && bits <= 8, "invalid bit stream geometry");
+    const uint8_t* p = in.take(stream_bytes(count, bits), what);   // fails before anything is allocated
     std::vector<uint8_t> out(static_cast<size_t>(count));
     for (int64_t i = 0; i < count; ++i) {
         const int64_t bit = i * bits;
@@ -155,6 +168,13 @@ std::unique_ptr<mfq_amd_tensor> load_nint(const uint8_t* blob, int64_t nbytes, i
     const int64_t ng = in.get<uint32_t>("NINT dimensions");
     MFQ_REQUIRE(out > 0 && ng > 0 && ng == (static_cast<int64_t>(neuron_len) + gs - 1) / gs,
                 "inconsistent NINT tensor dimensions");
+    // nothing is allocated from header counts the remaining bytes cannot back: two fp16 anchors per row, and at
+    // least one bit per group level, group minimum and code
+    in.need(checked_mul(out, 4, "NINT neuron metadata"), "NINT neuron metadata");
+    const int64_t level_count = checked_mul(out, ng, "NINT group metadata");
+    const int64_t values_per_row = checked_mul(ng, gs, "NINT row");
+    MFQ_REQUIRE(level_count / 4 <= in.left() && checked_mul(out, values_per_row, "NINT packed values") / 8 <= in.left(),
+                "truncated NINT payload");
     std::vector<float> scale(out), minimum(out);
     {
         const uint8_t* p = in.take(out * 2, "NINT neuron metadata");
@@ -195,7 +215,6 @@ std::unique_ptr<mfq_amd_tensor> load_nint(const uint8_t* blob, int64_t nbytes, i
     std::vector<uint8_t> row_bits(out);
     std::vector<int64_t> offsets(out);
     std::vector<uint8_t> packed;
-    const int64_t values_per_row = ng * gs;
     if (!per_row_widths) {
         const int64_t bytes = stream_bytes(out * values_per_row, bits);
         const uint8_t* p = in.take(bytes, "NINT packed values");
@@ -389,6 +408,8 @@ std::unique_ptr<mfq_amd_tensor> load_nvq(const uint8_t* blob, int64_t nbytes, in
         metadata = as_bytes(builtin_grid(d4 ? "d4_256" : "e8_256", e, d));
     }
     const int64_t ng = (neuron_len + 23) / 24, nvec = (neuron_len + dim - 1) / dim, nsign = (neuron_len + 7) / 8;
+    MFQ_REQUIRE(out > 0, "NVQ tensor has no rows");
+    in.need(checked_mul(out, 2, "NVQ neuron anchors"), "NVQ neuron anchors");
     std::vector<float> anchors(out);
     {
         const uint8_t* p = in.take(out * 2, "NVQ neuron anchors");
@@ -399,16 +420,19 @@ std::unique_ptr<mfq_amd_tensor> load_nvq(const uint8_t* blob, int64_t nbytes, in
             anchors[r] = half_to_float(a);
         }
     }
-    const int64_t state_bytes = stream_bytes(out * ng, sub_bits);
-    const int64_t index_bytes = stream_bytes(out * nvec, index_bits);
-    const int64_t sign_bytes = stream_bytes(out * nsign, 7);
+    const int64_t state_bytes = stream_bytes(checked_mul(out, ng, "NVQ state stream"), sub_bits);
+    const int64_t index_bytes = stream_bytes(checked_mul(out, nvec, "NVQ index stream"), index_bits);
+    const int64_t sign_bytes = stream_bytes(checked_mul(out, nsign, "NVQ sign stream"), 7);
+    // the streams (or the records they are rebuilt from) must be present before anything of their size is allocated
+    if (group64) in.need(checked_mul(checked_mul(out, ng, "NVQ group64 stream"), 8, "NVQ group64 stream"), "NVQ group64 stream");
+    else in.need(state_bytes + index_bytes + sign_bytes, "NVQ streams");
     std::vector<uint8_t> unpacked[3];   // states, indices, signs rebuilt from records
     const uint8_t *states, *indices, *signs;
     if (group64) {
         // record = state << 60 | three segments of 20 bits: 12-bit index, 7 sign bits and their parity
         // (cpp_runtime/backends/cuda/ops/vq.cpp:1319-1361); the runtime layout is the three streams
         const int64_t records = out * ng;
-        const uint8_t* p = in.take(records * 8, "NVQ group64 stream");
+        const uint8_t* p = in.take(checked_mul(records, 8, "NVQ group64 stream"), "NVQ group64 stream");
         unpacked[0].assign(static_cast<size_t>(state_bytes), 0);
         unpacked[1].assign(static_cast<size_t>(index_bytes), 0);
         unpacked[2].assign(static_cast<size_t>(sign_bytes), 0);
@@ -472,6 +496,7 @@ std::unique_ptr<mfq_amd_tensor> load_mxfp4(const uint8_t* blob, int64_t nbytes, 
     uint64_t dims[6];
     for (auto& d : dims) d = in.get<uint64_t>("MXFP4 header");
     MFQ_REQUIRE(version == 1 && kind == 4 && reserved == 0, "not an MXFP4 payload");
+    MFQ_REQUIRE(dims[0] <= (uint64_t(1) << 31) && dims[1] <= (uint64_t(1) << 31), "oversized MXFP4 geometry");
     const int64_t rows = static_cast<int64_t>(dims[0]), cols = static_cast<int64_t>(dims[1]);
     MFQ_REQUIRE(rows > 0 && cols > 0 && cols % 32 == 0 && dims[2] == dims[0] && dims[3] == dims[1] / 2 &&
                 dims[4] == dims[0] && dims[5] == dims[1] / 32, "inconsistent MXFP4 geometry");
@@ -595,6 +620,8 @@ int mfq_amd_mfe_load(const uint8_t* blob, int64_t nbytes, mfq_amd_mfe** out) {
             const uint64_t payload_len = in.get<uint64_t>("MFE pool header");
             const uint64_t runtime_len = short_pools ? 0 : in.get<uint64_t>("MFE pool header");
             MFQ_REQUIRE(count > 0 && (short_pools || dtype_len > 0) && dtype_len <= 32, "invalid MFE pool header");
+            MFQ_REQUIRE(count <= static_cast<uint32_t>(mfe->experts), "MFE pool lists more experts than the tensor has");
+            in.need(int64_t(count) * 4, "MFE expert ids");
             std::vector<int32_t> ids(count);
             std::memcpy(ids.data(), in.take(int64_t(count) * 4, "MFE expert ids"), size_t(count) * 4);
             for (int32_t e : ids) {
@@ -603,7 +630,9 @@ int mfq_amd_mfe_load(const uint8_t* blob, int64_t nbytes, mfq_amd_mfe** out) {
             }
             const std::string dtype = short_pools ? std::string("NINT")
                 : std::string(reinterpret_cast<const char*>(in.take(dtype_len, "MFE dtype")), dtype_len);
+            in.need_u64(runtime_len, "MFE runtime payload");
             (void)in.take(static_cast<int64_t>(runtime_len), "MFE runtime payload");
+            in.need_u64(payload_len, "MFE tensor payload");
             const uint8_t* payload = in.take(static_cast<int64_t>(payload_len), "MFE tensor payload");
             auto tensor = load_any(dtype, payload, static_cast<int64_t>(payload_len), mfe->out_per_expert);
             MFQ_REQUIRE(tensor->geom.local_experts == static_cast<int32_t>(count) &&

@@ -229,9 +229,10 @@ using namespace mfq_amd;
 
 extern "C" int mfq_amd_dequant(const mfq_amd_projection* proj, int32_t local_expert, float* out_dev, void* stream) {
     return guarded([&] {
-        MFQ_REQUIRE(proj && out_dev, "null argument");
+        MFQ_REQUIRE(proj, "null argument");
         const mfq_amd_projection p = canonical_projection(*proj);
         validate_projection(p, local_expert);
+        MFQ_REQUIRE(out_dev, "null argument");
         dev::DequantLaunch launch{p, local_expert, out_dev, as_stream(stream)};
         dev::dispatch_class(projection_class(p), launch);
         check_launch("dequant_kernel");

@@ -3,6 +3,7 @@
 // grouped projection entry point and the fused FFN object.
 #include "common.h"
 #include "decode.cuh"
+#include "device_state.h"
 #include "fast_rows.cuh"
 #include "launch.cuh"
 #include "moe_args.h"
@@ -11,6 +12,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <vector>
 
 namespace mfq_amd {
@@ -363,8 +365,6 @@ void launch_rows_exact(const RowsArgs& args, int slots, const int* present, cons
     }
 }
 
-namespace {
-
 // IEEE binary64 -> binary16 with one rounding (the reference's half type converts a double directly).
 uint16_t double_to_half(double value) {
     uint64_t u;
@@ -403,12 +403,19 @@ float half_to_float_host(uint16_t h) {
     return sign ? -v : v;
 }
 
+namespace {
+
 template <class T>
 T* device_alloc(size_t count) {
     void* p = nullptr;
     MFQ_HIP(hipMalloc(&p, sizeof(T) * (count ? count : 1)));
     return static_cast<T*>(p);
 }
+
+constexpr int kMaxDevices = 64;
+std::mutex g_state_mutex;
+DeviceState g_states[kMaxDevices];
+bool g_state_ready[kMaxDevices];
 
 // Device-side tables of a set of pools: descriptors, kernel classes, per-expert bytes.
 struct PoolTables {
@@ -446,9 +453,42 @@ struct PoolTables {
 };
 
 }  // namespace
+
+const DeviceState& device_state() {
+    int device = 0;
+    MFQ_HIP(hipGetDevice(&device));
+    MFQ_REQUIRE(device >= 0 && device < kMaxDevices, "device index out of range");
+    std::lock_guard<std::mutex> lock(g_state_mutex);
+    if (!g_state_ready[device]) {
+        std::vector<uint16_t> table(65536);
+        for (uint32_t h = 0; h < 65536; ++h) {
+            const double g = static_cast<double>(half_to_float_host(static_cast<uint16_t>(h)));
+            table[h] = double_to_half(1.0 / (1.0 + std::exp(-g)));
+        }
+        uint16_t* sigmoid = device_alloc<uint16_t>(65536);   // lives until the process ends
+        MFQ_HIP(hipMemcpy(sigmoid, table.data(), sizeof(uint16_t) * 65536, hipMemcpyHostToDevice));
+        raise_routing_limits();
+        raise_prefill_limits();
+        g_states[device].sigmoid_table = sigmoid;
+        g_state_ready[device] = true;
+    }
+    return g_states[device];
+}
+
 }  // namespace mfq_amd
 
 using namespace mfq_amd;
+
+extern "C" int mfq_amd_init(void) {
+    return guarded([&] { (void)device_state(); });
+}
+
+extern "C" int32_t mfq_amd_moe_ffn_decode_limit(int32_t requested, int32_t top_k) {
+    if (top_k < 1) return 0;
+    const int32_t limit = requested > 0 ? requested : 32;
+    const int32_t most = kPlanThreads / top_k;    // a decode plan is one thread per routed pair
+    return limit < most ? limit : most;
+}
 
 struct mfq_amd_moe_ffn {
     mfq_amd_moe_ffn_config config{};
@@ -464,7 +504,8 @@ struct mfq_amd_moe_ffn {
             *d_tile_offsets = nullptr, *d_counts = nullptr, *d_bounds = nullptr, *d_tile_bounds = nullptr,
             *d_tile_experts = nullptr, *d_ids_dst = nullptr, *d_distinct = nullptr;
     int64_t* d_touched = nullptr;
-    uint16_t *d_gu = nullptr, *d_hidden = nullptr, *d_pairs = nullptr, *d_sigmoid = nullptr;
+    uint16_t *d_gu = nullptr, *d_hidden = nullptr, *d_pairs = nullptr;
+    const uint16_t* d_sigmoid = nullptr;   // the device's table: not owned
     int32_t* d_wave_base = nullptr;      // scratch of the two-kernel route plan
     int32_t* d_route_ids = nullptr;      // routes selected by run_logits
     float* d_route_weights = nullptr;
@@ -480,7 +521,7 @@ struct mfq_amd_moe_ffn {
     ~mfq_amd_moe_ffn() {
         void* all[] = {d_pools, d_pool_class, d_pool_bytes, d_expert_pool, d_expert_info, d_item_info, d_pair_items, d_items, d_class_offsets, d_tile_items,
                        d_tile_offsets, d_counts, d_bounds, d_tile_bounds, d_tile_experts, d_ids_dst, d_distinct,
-                       d_touched, d_gu, d_hidden, d_pairs, d_sigmoid, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base};
+                       d_touched, d_gu, d_hidden, d_pairs, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base};
         for (void* p : all) if (p) (void)hipFree(p);
         for (hipEvent_t e : events) if (e) (void)hipEventDestroy(e);
     }
@@ -506,7 +547,7 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
         MFQ_REQUIRE(c.gate.experts <= kPlanMaxExperts, "at most 1024 experts");
         f->experts = c.gate.experts; f->hidden = c.gate.neuron_len; f->intermediate = c.gate.out_per_expert;
         f->top_k = c.top_k; f->max_tokens = c.max_tokens;
-        f->decode_limit = c.decode_token_limit > 0 ? c.decode_token_limit : 32;
+        f->decode_limit = mfq_amd_moe_ffn_decode_limit(c.decode_token_limit, c.top_k);
         f->tables.add_slot(0, c.gate);
         f->tables.add_slot(1, c.up);
         f->tables.add_slot(2, c.down);
@@ -573,7 +614,7 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
         f->d_gu = device_alloc<uint16_t>(pairs * 2 * f->intermediate);
         f->d_hidden = device_alloc<uint16_t>(pairs * f->intermediate);
         f->d_pairs = device_alloc<uint16_t>(pairs * f->hidden);
-        f->d_sigmoid = device_alloc<uint16_t>(65536);
+        f->d_sigmoid = device_state().sigmoid_table;
         f->d_route_ids = device_alloc<int32_t>(pairs);
         f->d_route_weights = device_alloc<float>(pairs);
         f->d_wave_base = device_alloc<int32_t>(static_cast<size_t>(kPlanThreads / 64) * E);
@@ -597,12 +638,6 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
             if (rows_fast_geometry(f->intermediate, MFQ_AMD_F16))
                 f->d_hidden_packed = device_alloc<uint32_t>(decode_tokens * c.top_k * dev::xpack_row_dwords(f->intermediate));
         }
-        std::vector<uint16_t> table(65536);
-        for (uint32_t h = 0; h < 65536; ++h) {
-            const double g = static_cast<double>(half_to_float_host(static_cast<uint16_t>(h)));
-            table[h] = double_to_half(1.0 / (1.0 + std::exp(-g)));
-        }
-        MFQ_HIP(hipMemcpy(f->d_sigmoid, table.data(), sizeof(uint16_t) * 65536, hipMemcpyHostToDevice));
         MFQ_HIP(hipMemset(f->d_gu, 0, sizeof(uint16_t) * pairs * 2 * f->intermediate));
         MFQ_HIP(hipMemset(f->d_pairs, 0, sizeof(uint16_t) * pairs * f->hidden));
         MFQ_HIP(hipDeviceSynchronize());
@@ -685,9 +720,6 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         auto rows_per_block = [&](int out_rows, int slots) {
             int rows = 256;
             const int least = rows_fast_min_block(rows_in_width);
-            // measurement aid: MFQ_AMD_ROWS_PER_BLOCK (read once per process) overrides the choice below
-            static const int forced = [] { const char* text = std::getenv("MFQ_AMD_ROWS_PER_BLOCK"); return text ? std::atoi(text) : 0; }();
-            if (forced > 0) return forced / least * least > 0 ? forced / least * least : least;
             while (rows > least && static_cast<int64_t>(pairs) * slots * ((out_rows + rows - 1) / rows) < 2048) rows /= 2;
             return rows;
         };
@@ -1004,14 +1036,7 @@ extern "C" int mfq_amd_swiglu(const void* gate_f16_dev, const void* up_f16_dev, 
     return guarded([&] {
         MFQ_REQUIRE(gate_f16_dev && up_f16_dev && hidden_f16_dev && count >= 0, "invalid argument");
         if (!count) return;
-        static uint16_t* table = nullptr;
-        if (swiglu_limit <= 0.0f && !table) {
-            std::vector<uint16_t> host(65536);
-            for (uint32_t h = 0; h < 65536; ++h)
-                host[h] = double_to_half(1.0 / (1.0 + std::exp(-static_cast<double>(half_to_float_host(static_cast<uint16_t>(h))))));
-            MFQ_HIP(hipMalloc(reinterpret_cast<void**>(&table), sizeof(uint16_t) * 65536));
-            MFQ_HIP(hipMemcpy(table, host.data(), sizeof(uint16_t) * 65536, hipMemcpyHostToDevice));
-        }
+        const uint16_t* table = device_state().sigmoid_table;
         hipLaunchKernelGGL(dev::swiglu_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0,
                            as_stream(stream), static_cast<const uint16_t*>(gate_f16_dev),
                            static_cast<const uint16_t*>(up_f16_dev), count, count, count,

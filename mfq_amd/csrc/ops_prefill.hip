@@ -14,6 +14,7 @@
 // and geometries the streaming kernel does not serve.
 #include "common.h"
 #include "decode.cuh"
+#include "device_state.h"
 #include "fast.cuh"
 #include "launch.cuh"
 #include "moe_args.h"
@@ -131,6 +132,7 @@ constexpr int kOutPitch = 2 * kFastTileN + 16;      // bytes per pair of the out
 // what the tables of the pool leave of their region plus kSideExtraBytes, for runs of up to
 // kSideMaxRun steps.
 constexpr int kSideExtraBytes = 7168;
+constexpr int kTilesFastLdsBytes = kFastLdsBytes + kNvqFastLdsBytes + kSideExtraBytes + kPrefillTileM * 4;   // dynamic LDS of the tile kernel
 constexpr int kSideMaxRun = 8;
 constexpr int kLevelWindow = 64;
 constexpr int kLevelPitch = kLevelWindow + 4;
@@ -718,6 +720,15 @@ struct TilesLaunch {
 
 }  // namespace dev
 
+void raise_prefill_limits() {
+    MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::moe_tiles_fast_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, dev::kTilesFastLdsBytes));
+    MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::moe_tiles_fast_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, dev::kTilesFastLdsBytes));
+    MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::swiglu_tiles_lds_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, dev::kSigmoidTableBytes));
+}
+
 bool tiles_fast_geometry(int in_width, int in_dtype, int in_vector_ok) {
     return in_width % dev::kLaneColumns == 0 && in_width >= 2 * dev::kLaneColumns && in_dtype != MFQ_AMD_F32 && in_vector_ok != 0;
 }
@@ -730,15 +741,8 @@ void launch_tiles_fast(const RowsArgs& args, int slots, int max_tiles, bool nvq,
     const int row_blocks = (args.out_rows + dev::kFastTileN - 1) / dev::kFastTileN;
     const dim3 grid((max_tiles + 7) / 8 * 8 * row_blocks * slots);
     (void)nvq;   // the table region also holds the NINT level windows
-    const int bytes = dev::kFastLdsBytes + dev::kNvqFastLdsBytes + dev::kSideExtraBytes + kPrefillTileM * 4;
-    static bool raised = false;   // more than the default 64 KB of dynamic LDS
-    if (!raised) {
-        MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::moe_tiles_fast_kernel<true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
-        MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::moe_tiles_fast_kernel<false>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
-        raised = true;
-    }
+    const int bytes = dev::kTilesFastLdsBytes;   // more than the default 64 KB of dynamic LDS: raised by device_state()
+    (void)device_state();
     if (a.in_tiles != nullptr) hipLaunchKernelGGL(dev::moe_tiles_fast_kernel<true>, grid, dim3(256), bytes, stream, a);
     else hipLaunchKernelGGL(dev::moe_tiles_fast_kernel<false>, grid, dim3(256), bytes, stream, a);
     check_launch("moe_tiles_fast_kernel");
@@ -762,12 +766,7 @@ void launch_swiglu_tiles(const uint16_t* gate, const uint16_t* up, int64_t gate_
     const int64_t items = static_cast<int64_t>(pairs) * (inner / dev::kLaneColumns);
     constexpr int kResidentBlocks = 256;    // one per CU: the table takes 128 KB of a CU's 160 KB of LDS
     if (limit <= 0.0f && items >= static_cast<int64_t>(kResidentBlocks) * 1024 * 2 && reinterpret_cast<uintptr_t>(table) % 16 == 0) {
-        static bool raised = false;
-        if (!raised) {
-            MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::swiglu_tiles_lds_kernel),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, dev::kSigmoidTableBytes));
-            raised = true;
-        }
+        (void)device_state();   // the kernel's dynamic-LDS limit is raised there
         hipLaunchKernelGGL(dev::swiglu_tiles_lds_kernel, dim3(kResidentBlocks), dim3(1024), dev::kSigmoidTableBytes, stream, gate, up,
                            gate_stride, inner, pairs, table, ids, down_info, experts, hidden);
         check_launch("swiglu_tiles_lds_kernel");

@@ -1,6 +1,7 @@
 // Routing: reproducible router logits, softmax top-k, and the pair-by-expert route plan.
 #include "common.h"
 #include "decode.cuh"
+#include "device_state.h"
 #include "plan.h"
 #include "xpack.cuh"
 
@@ -322,13 +323,16 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
     const int pair_scan = block_inclusive_scan(tid < E ? count : 0, scratch);
     const int route_tiles = tid < E ? (count + a.tile_m - 1) / a.tile_m : 0;
     const int tile_scan = block_inclusive_scan(route_tiles, scratch);
+    const bool want_route_tiles = a.tile_bounds != nullptr && a.tile_experts != nullptr;
     if (tid < E) {
         start[tid] = pair_scan - count;
         a.expert_bounds[tid + 1] = pair_scan;
-        a.tile_bounds[tid + 1] = tile_scan;
-        for (int t = tile_scan - route_tiles; t < tile_scan; ++t) a.tile_experts[t] = tid;
+        if (want_route_tiles) {
+            a.tile_bounds[tid + 1] = tile_scan;
+            for (int t = tile_scan - route_tiles; t < tile_scan; ++t) a.tile_experts[t] = tid;
+        }
     }
-    if (tid == 0) { a.expert_bounds[0] = 0; a.tile_bounds[0] = 0; }
+    if (tid == 0) { a.expert_bounds[0] = 0; if (want_route_tiles) a.tile_bounds[0] = 0; }
     __syncthreads();
 
     if (a.wave_base != nullptr) {
@@ -722,17 +726,19 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_small_kernel(PlanArgs
 
 }  // namespace dev
 
+void raise_routing_limits() {
+    MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::route_plan_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::route_scatter_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024));
+}
+
 void launch_route_plan(const PlanArgs& args, hipStream_t stream) {
     MFQ_REQUIRE(args.experts > 0 && args.experts <= kPlanMaxExperts, "route plan supports 1..1024 experts");
     MFQ_REQUIRE(args.pairs >= 0 && args.tile_m > 0, "invalid route plan geometry");
     const size_t lds = sizeof(int) * (static_cast<size_t>(kPlanThreads / 64) * args.experts + 2 * args.experts +
                                       kPlanThreads / 64 + 2 * dev::K_CLASS_COUNT * (kPlanThreads / 64) + 8);
-    static bool raised = false;
-    if (lds > 64 * 1024 && !raised) {
-        MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::route_plan_kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-        raised = true;
-    }
+    if (lds > 64 * 1024) (void)device_state();   // the kernel's dynamic-LDS limit is raised there
     const int pack_rows = args.pack.src != nullptr ? args.pack.rows : 0;
     MFQ_REQUIRE(pack_rows == 0 || (args.pack.width % dev::kLaneColumns == 0 && args.pack.width <= dev::kLaneColumns * kPlanThreads),
                 "activation width cannot be packed");
@@ -764,12 +770,7 @@ void launch_route_plan(const PlanArgs& args, hipStream_t stream) {
     check_launch("route_plan_kernel");
     if (args.wave_base != nullptr) {
         const size_t scatter_lds = sizeof(int) * 2 * (kPlanThreads / 64) * args.experts;
-        static bool scatter_raised = false;
-        if (scatter_lds > 64 * 1024 && !scatter_raised) {
-            MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::route_scatter_kernel),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024));
-            scatter_raised = true;
-        }
+        if (scatter_lds > 64 * 1024) (void)device_state();
         hipLaunchKernelGGL(dev::route_scatter_kernel, dim3(kPlanThreads / 64), dim3(kPlanThreads), scatter_lds, stream, args);
         check_launch("route_scatter_kernel");
     }

@@ -342,3 +342,125 @@ def test_null_arguments_return_invalid():
     assert lib.mfq_amd_topk(None, 0, 1, 8, 2, 1, 1e-20, 1.0, None, None, None) == L.ERR_INVALID
     assert lib.mfq_amd_grouped_matmul_workspace(4, 2, 8) > 0
     assert lib.mfq_amd_grouped_matmul_workspace(-1, 2, 8) == 0
+
+
+# ------------------------------------------------------------------ hostile lengths ----
+def _nint_header(out, ng, neuron_len, gs=24, bits=4, sub=6):
+    import struct
+    return struct.pack("<BBiiiI", bits | 0x80, sub, gs, 0, neuron_len, 2) + struct.pack("<qq", out, neuron_len) + \
+        struct.pack("<II", out, ng)
+
+
+def test_blobs_with_huge_counts_are_rejected_before_anything_is_allocated():
+    """Header counts the remaining bytes cannot back must fail as a status code: a 40-byte NINT blob that names
+    2^32 - 1 rows, an NVQ blob with 2^32 - 1 rows, an MXFP4 blob whose dimensions overflow the byte count."""
+    import struct
+    status, _ = _load("NINT", _nint_header(0xFFFFFFFF, 4, 96) + b"\0" * 8)
+    assert status == L.ERR_INVALID, L.lib().mfq_amd_last_error()
+    status, _ = _load("NINT", _nint_header(0xFFFFFFFF, 0xFFFFFFFF, 96) + b"\0" * 8)
+    assert status == L.ERR_INVALID
+    # rows x groups fits, but the code stream does not
+    status, _ = _load("NINT", _nint_header(1 << 20, 4, 96) + b"\0" * (4 << 20) + b"\0" * 64)
+    assert status == L.ERR_INVALID and b"truncated" in L.lib().mfq_amd_last_error()
+    rng = np.random.default_rng(2)
+    good = bytearray(nvq.pack_nvq(nvq_quant.random_nvq(4, 96, nvq.NVQ3_D4, rng)))
+    rows_at = 20 + 16
+    assert struct.unpack_from("<I", good, rows_at)[0] == 4
+    struct.pack_into("<I", good, rows_at, 0xFFFFFFFF)
+    struct.pack_into("<q", good, 20, 0xFFFFFFFF)
+    status, _ = _load("NVQ", bytes(good))
+    assert status == L.ERR_INVALID and b"truncated" in L.lib().mfq_amd_last_error()
+    mxb = bytearray(mx.pack_mx(mx.random_mxfp4(2, 32, rng)))
+    for rows, cols in ((1 << 62, 32), (1 << 40, 1 << 40), ((1 << 63) + 2, 32)):
+        struct.pack_into("<6Q", mxb, 8, rows, cols, rows, cols // 2, rows, cols // 32)
+        status, _ = _load("MXFP4", bytes(mxb))
+        assert status == L.ERR_INVALID, (rows, cols)
+
+
+@pytest.mark.parametrize("payload_len,runtime_len", [((1 << 63) - 1, 0), ((1 << 64) - 1, 0), (0, (1 << 63) - 8),
+                                                     ((1 << 63) - 40, 64), (1 << 62, 1 << 62)])
+def test_mfe_lengths_near_the_top_of_the_range_do_not_wrap(payload_len, runtime_len):
+    """payload_len / runtime_len are unsigned 64-bit fields: a value near INT64_MAX must not pass the bounds check
+    by overflowing offset + length (cpp_runtime/backends/cuda/ops/moe.cpp:70-87 compares against the bytes left)."""
+    import struct
+    rng = np.random.default_rng(4)
+    payload = nint.pack_nint(nint_quant.random_codes(4, 48, nint.NintSpec(4, 24, 6), rng))
+    head = struct.pack("<4sIIII", b"MFE1", 1, 4, 48, 1)
+    blob = head + struct.pack("<IIQQ", 1, 4, payload_len, runtime_len) + np.asarray([0], "<i4").tobytes() + b"NINT" + payload
+    status, _ = _mfe_status(blob)
+    assert status == L.ERR_INVALID and b"truncated" in L.lib().mfq_amd_last_error()
+
+
+def test_mfe_pool_with_more_experts_than_the_tensor_is_rejected():
+    import struct
+    blob = struct.pack("<4sIIII", b"MFE1", 2, 4, 48, 1) + struct.pack("<IIQQ", 0xFFFFFFF0, 4, 16, 0) + b"\0" * 64
+    status, _ = _mfe_status(blob)
+    assert status == L.ERR_INVALID
+
+
+@pytest.mark.parametrize("cut", [1, 9, 40, 200])
+@pytest.mark.parametrize("family", ["NVQ", "NVQJ", "MXFP4", "MFE"])
+def test_truncated_blobs_of_every_family_are_rejected(family, cut):
+    rng = np.random.default_rng(13)
+    if family == "NVQ":
+        blob, load = nvq.pack_nvq(nvq_quant.random_nvq(4, 96, nvq.NVQ3_D4, rng)), lambda b: _load("NVQ", b)[0]
+    elif family == "NVQJ":
+        blob, load = nvq.pack_nvq(nvq_quant.random_nvq_jsc(4, 96, nvq.NVQ3_D4_1024, rng)), lambda b: _load("NVQ", b)[0]
+    elif family == "MXFP4":
+        blob, load = mx.pack_mx(mx.random_mxfp4(4, 64, rng)), lambda b: _load("MXFP4", b)[0]
+    else:
+        pools = [MFE.MfePool(np.array([0, 1], dtype=np.int32), nint_quant.random_codes(8, 96, nint.NintSpec(4, 24, 6), rng))]
+        blob, load = MFE.pack_mfe(MFE.MfeTensor((2, 4, 96), pools)), lambda b: _mfe_status(b)[0]
+    assert load(blob) == 0
+    assert load(blob[:-cut]) == L.ERR_INVALID
+    assert load(blob[:min(cut, len(blob) - 1)]) == L.ERR_INVALID
+    assert load(blob + b"\0") == L.ERR_INVALID
+
+
+# --------------------------------------------------------------- descriptor checks ----
+def _nint_view(rng, rows=8, width=96, bits=4, gs=24, out_per_expert=4):
+    t = nint_quant.random_codes(rows, width, nint.NintSpec(bits, gs, 6), rng)
+    status, handle = _load("NINT", nint.pack_nint(t), out_per_expert)
+    assert status == 0
+    view = L.Projection()
+    assert L.lib().mfq_amd_tensor_host_view(handle, C.byref(view)) == 0
+    return view, handle
+
+
+def test_nint_descriptor_with_short_stream_or_stride_is_rejected():
+    """The checks of the reference's validate() (cpp_runtime/backends/cpu/ops/packed_nint.cpp:15-34) a host can make
+    without reading device memory: the last expert's rows fit the stream, an expert's rows fit its stride, and the
+    code width is 0..8.  Validation runs before any device call, so this needs no GPU."""
+    rng = np.random.default_rng(17)
+    lib = L.lib()
+    view, handle = _nint_view(rng)
+    stream = 4 * view.groups * view.group_size * 4 // 8
+
+    def status_of(v):
+        return lib.mfq_amd_dequant(C.byref(v), 0, None, None)
+
+    bad = L.Projection.from_buffer_copy(view); bad.sizes[0] = view.q_expert_stride + stream - 1
+    assert status_of(bad) == L.ERR_INVALID and b"exceeds storage" in lib.mfq_amd_last_error()
+    bad = L.Projection.from_buffer_copy(view); bad.q_expert_stride = stream - 1
+    assert status_of(bad) == L.ERR_INVALID and b"stride" in lib.mfq_amd_last_error()
+    bad = L.Projection.from_buffer_copy(view); bad.uniform_bits = 9
+    assert status_of(bad) == L.ERR_INVALID and b"width" in lib.mfq_amd_last_error()
+    bad = L.Projection.from_buffer_copy(view); bad.uniform_bits = 0; bad.sizes[0] = view.q_expert_stride + stream // 4 - 1
+    assert status_of(bad) == L.ERR_INVALID                       # per-row widths: at least one bit per code
+    ok = L.Projection.from_buffer_copy(view); ok.sizes[0] = view.q_expert_stride + stream
+    assert status_of(ok) == L.ERR_INVALID and b"null" in lib.mfq_amd_last_error()   # passes validation; out is null
+    lib.mfq_amd_tensor_free(handle)
+
+
+def test_decode_token_limit_is_clamped_to_one_thread_per_pair():
+    lib = L.lib()
+    assert lib.mfq_amd_moe_ffn_decode_limit(0, 10) == 32
+    assert lib.mfq_amd_moe_ffn_decode_limit(128, 10) == 102          # 1024 threads / 10 routes
+    assert lib.mfq_amd_moe_ffn_decode_limit(128, 8) == 128
+    assert lib.mfq_amd_moe_ffn_decode_limit(4096, 1) == 1024
+    assert lib.mfq_amd_moe_ffn_decode_limit(64, 32) == 32
+    assert lib.mfq_amd_moe_ffn_decode_limit(16, 0) == 0
+    for top_k in range(1, 33):
+        for requested in (0, 1, 31, 32, 33, 128, 1024, 100000):
+            limit = lib.mfq_amd_moe_ffn_decode_limit(requested, top_k)
+            assert 1 <= limit and limit * top_k <= 1024
