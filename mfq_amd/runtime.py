@@ -166,6 +166,17 @@ class MixedMoeRuntime:
         self.struct = L.MoeTensor(self._views, len(self.pools), self.experts, self.out_per_expert, self.neuron_len)
 
     @classmethod
+    def from_dense(cls, tensor) -> "MixedMoeRuntime":
+        """A single dense matrix as a one-expert tensor (no expert map): how a shared expert is handed to the FFN."""
+        self = cls.__new__(cls)
+        packed = PackedTensor.from_tensor(tensor, 0).cuda()
+        self.experts, self.out_per_expert, self.neuron_len = 1, packed.view.output_rows, packed.view.input_width
+        self.pools = [packed]
+        self._views = (L.Projection * 1)(packed.view)
+        self.struct = L.MoeTensor(self._views, 1, 1, self.out_per_expert, self.neuron_len)
+        return self
+
+    @classmethod
     def from_blob(cls, blob: bytes) -> "MixedMoeRuntime":
         """Through the C++ MFE container reader instead of the Python object model."""
         self = cls.__new__(cls)

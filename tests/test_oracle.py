@@ -346,6 +346,34 @@ def test_swiglu_rounding_chain():
     assert np.array_equal(got, expect.view(np.uint16))
 
 
+def test_clamped_swiglu_branch():
+    """swiglu_limit > 0 (mfq/kernels/cuda/mfe_ffn.h:111-114): g' = min(g, L) (no lower clip), u' = clip(u, -L, L),
+    half((g' / (1 + expf(-g'))) * u') in fp32.  Pinned by a float32 numpy closed form to one fp16 step (expf of two
+    libraries), and exactly by what the clips imply: an operand beyond the limit gives the result of the limit itself."""
+    rng = np.random.default_rng(24)
+    g = rng.normal(0, 4, 6000).astype(np.float16)
+    u = rng.normal(0, 4, 6000).astype(np.float16)
+    one = lambda a, b, limit: O.lib().orc_swiglu_f16(int(np.float16(a).view(np.uint16)), int(np.float16(b).view(np.uint16)), limit)
+    for limit in (7.0, 1.5, 0.25):
+        L = np.float32(limit)
+        gc = np.minimum(g.astype(np.float32), L)
+        uc = np.clip(u.astype(np.float32), -L, L)
+        act = (gc / (np.float32(1.0) + np.exp(-gc, dtype=np.float32))).astype(np.float32)
+        expect = (act * uc).astype(np.float32).astype(np.float16)
+        got = O.swiglu_array(g, u, limit)
+        a, b = got.view(np.uint16).astype(np.int32), expect.view(np.uint16).astype(np.int32)
+        assert np.all(np.abs(a - b) <= 1) and np.mean(a == b) > 0.99
+        # the clips, exactly
+        assert one(60.0, 3.0, limit) == one(limit, 3.0, limit)
+        assert one(2.0, 900.0, limit) == one(2.0, limit, limit) and one(2.0, -900.0, limit) == one(2.0, -limit, limit)
+        # no lower clip of the gate: a very negative gate gives (nearly) zero, not -limit * sigmoid(-limit) * u
+        assert abs(float(np.uint16(one(-30.0, 1.0, limit)).view(np.float16))) < 1e-6
+        # inside the limits it is plain SiLU(g) * u in fp32, one rounding: differs from the table chain only by roundings
+        assert one(0.125, 0.125, limit) == one(0.125, 0.125, 1000.0)
+    # limit <= 0 selects the table chain
+    assert one(1.0, 2.0, 0.0) == one(1.0, 2.0, -1.0)
+
+
 def test_expert_ffn_composition():
     rng = np.random.default_rng(15)
     gate = O.Projection(O.nint_runtime(QN.random_codes(32, 96, FN.NINT4, rng)))
