@@ -243,6 +243,18 @@ int mfq_amd_grouped_matmul(const mfq_amd_moe_tensor* tensor, const void* x_dev, 
                            int32_t x_rows_per_token, const int32_t* ids_dev, int32_t tokens, int32_t top_k,
                            void* out_f16_dev, void* workspace_dev, int64_t workspace_bytes, void* stream);
 
+/* The same projection without a workspace argument and without any allocation, for callers that cannot allocate
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  The route plan lives in a static device array of mfq_amd_grouped_matmul_static_capacity() bytes
+ * (128 KiB per GPU, held until the process ends): calls whose mfq_amd_grouped_matmul_workspace(tokens, top_k,
+ * experts) exceeds it return MFQ_AMD_ERR_INVALID.  mfq_amd_init() must have run on the device (it allocates; this
+ * entry point does not).  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams,
+ * or two graphs replayed at the same time) race; calls on one stream are ordered and safe. */
+int64_t mfq_amd_grouped_matmul_static_capacity(void);
+int mfq_amd_grouped_matmul_static(const mfq_amd_moe_tensor* tensor, const void* x_dev, int32_t x_dtype,
+                                  int32_t x_rows_per_token, const int32_t* ids_dev, int32_t tokens, int32_t top_k,
+                                  void* out_f16_dev, void* stream);
+
 /* hidden = swiglu(gate, up) with the reference's fp16 rounding chain
  * (mfq/kernels/cuda/mfe_ffn.h:105-118; cuda/storage/moe_ffn_pipeline.cpp:154-169).  Uses the device's sigmoid
  * table (see mfq_amd_init). */

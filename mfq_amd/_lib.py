@@ -89,6 +89,9 @@ EXPORTS = {
     "mfq_amd_grouped_matmul_workspace": (C.c_int64, [C.c_int32, C.c_int32, C.c_int32]),
     "mfq_amd_grouped_matmul": (C.c_int, [C.POINTER(MoeTensor), C.c_void_p, C.c_int32, C.c_int32, C.c_void_p,
                                          C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
+    "mfq_amd_grouped_matmul_static_capacity": (C.c_int64, []),
+    "mfq_amd_grouped_matmul_static": (C.c_int, [C.POINTER(MoeTensor), C.c_void_p, C.c_int32, C.c_int32, C.c_void_p,
+                                                C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]),
     "mfq_amd_swiglu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_float, C.c_void_p, C.c_void_p]),
     "mfq_amd_weighted_reduce_shared_gate": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                                      C.c_int32, C.c_void_p, C.c_void_p]),

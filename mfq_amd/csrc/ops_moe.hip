@@ -13,6 +13,7 @@
 #include <cstring>
 #include <memory>
 #include <mutex>
+#include <string>
 #include <vector>
 
 namespace mfq_amd {
@@ -412,6 +413,12 @@ T* device_alloc(size_t count) {
     return static_cast<T*>(p);
 }
 
+// Scratch memory of mfq_amd_grouped_matmul_static: one copy per device that loads the library, held until the
+// process ends.  In host code the name stands for the symbol, not for device memory: its per-device address comes
+// from hipGetSymbolAddress (device_state()) and only that address is handed to kernels.
+constexpr int64_t kStaticScratchBytes = 128 * 1024;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 constexpr int kMaxDevices = 64;
 std::mutex g_state_mutex;
 DeviceState g_states[kMaxDevices];
@@ -469,10 +476,22 @@ const DeviceState& device_state() {
         MFQ_HIP(hipMemcpy(sigmoid, table.data(), sizeof(uint16_t) * 65536, hipMemcpyHostToDevice));
         raise_routing_limits();
         raise_prefill_limits();
+        void* scratch_at = nullptr;
+        MFQ_HIP(hipGetSymbolAddress(&scratch_at, HIP_SYMBOL(scratch)));
+        MFQ_REQUIRE(scratch_at != nullptr && reinterpret_cast<uintptr_t>(scratch_at) % 256 == 0, "static scratch array has no usable device address");
+        g_states[device].static_scratch = scratch_at;
         g_states[device].sigmoid_table = sigmoid;
         g_state_ready[device] = true;
     }
     return g_states[device];
+}
+
+const DeviceState* device_state_if_ready() {
+    int device = 0;
+    MFQ_HIP(hipGetDevice(&device));
+    MFQ_REQUIRE(device >= 0 && device < kMaxDevices, "device index out of range");
+    std::lock_guard<std::mutex> lock(g_state_mutex);
+    return g_state_ready[device] ? &g_states[device] : nullptr;
 }
 
 }  // namespace mfq_amd
@@ -937,10 +956,11 @@ extern "C" int64_t mfq_amd_grouped_matmul_workspace(int32_t tokens, int32_t top_
     return grouped_layout(tokens, top_k, experts).total;
 }
 
-extern "C" int mfq_amd_grouped_matmul(const mfq_amd_moe_tensor* tensor, const void* x_dev, int32_t x_dtype,
-                                      int32_t x_rows_per_token, const int32_t* ids_dev, int32_t tokens, int32_t top_k,
-                                      void* out_f16_dev, void* workspace_dev, int64_t workspace_bytes, void* stream_ptr) {
-    return guarded([&] {
+namespace {
+void grouped_matmul(const mfq_amd_moe_tensor* tensor, const void* x_dev, int32_t x_dtype, int32_t x_rows_per_token,
+                    const int32_t* ids_dev, int32_t tokens, int32_t top_k, void* out_f16_dev, void* workspace_dev,
+                    int64_t workspace_bytes, void* stream_ptr) {
+    {
         MFQ_REQUIRE(tensor && x_dev && ids_dev && out_f16_dev && workspace_dev, "null argument");
         MFQ_REQUIRE(tokens >= 0 && top_k >= 1, "invalid route geometry");
         MFQ_REQUIRE(x_rows_per_token == 1 || x_rows_per_token == top_k, "x must be [tokens, K] or [tokens, routes, K]");
@@ -1028,6 +1048,36 @@ extern "C" int mfq_amd_grouped_matmul(const mfq_amd_moe_tensor* tensor, const vo
         bool any = false;
         for (int c = 0; c < dev::K_CLASS_COUNT; ++c) any = any || (fast ? tables.exact_present[0][c] : tables.present[0][c]);
         if (any) launch_rows_exact(rows, 1, fast ? tables.exact_present[0] : tables.present[0], bound, stream);
+    }
+}
+}  // namespace
+
+extern "C" int mfq_amd_grouped_matmul(const mfq_amd_moe_tensor* tensor, const void* x_dev, int32_t x_dtype,
+                                      int32_t x_rows_per_token, const int32_t* ids_dev, int32_t tokens, int32_t top_k,
+                                      void* out_f16_dev, void* workspace_dev, int64_t workspace_bytes, void* stream_ptr) {
+    return guarded([&] {
+        grouped_matmul(tensor, x_dev, x_dtype, x_rows_per_token, ids_dev, tokens, top_k, out_f16_dev, workspace_dev,
+                       workspace_bytes, stream_ptr);
+    });
+}
+
+extern "C" int64_t mfq_amd_grouped_matmul_static_capacity(void) { return kStaticScratchBytes; }
+
+extern "C" int mfq_amd_grouped_matmul_static(const mfq_amd_moe_tensor* tensor, const void* x_dev, int32_t x_dtype,
+                                             int32_t x_rows_per_token, const int32_t* ids_dev, int32_t tokens,
+                                             int32_t top_k, void* out_f16_dev, void* stream_ptr) {
+    return guarded([&] {
+        MFQ_REQUIRE(tensor, "null argument");
+        MFQ_REQUIRE(tokens >= 0 && top_k >= 1 && tensor->experts > 0, "invalid route geometry");
+        const int64_t needed = mfq_amd_grouped_matmul_workspace(tokens, top_k, tensor->experts);
+        if (needed > kStaticScratchBytes)
+            fail_invalid("route plan of " + std::to_string(needed) + " bytes exceeds the static scratch of " +
+                         std::to_string(kStaticScratchBytes) + " bytes: use mfq_amd_grouped_matmul with a workspace");
+        const DeviceState* state = device_state_if_ready();
+        MFQ_REQUIRE(state != nullptr, "mfq_amd_init() must have run on this device before the allocation-free entry point");
+        // every plan list is written before it is read, so nothing of the previous call's contents needs clearing
+        grouped_matmul(tensor, x_dev, x_dtype, x_rows_per_token, ids_dev, tokens, top_k, out_f16_dev, state->static_scratch,
+                       kStaticScratchBytes, stream_ptr);
     });
 }
 
