@@ -223,7 +223,8 @@ int mfq_amd_moe_ffn_routes(mfq_amd_moe_ffn* ffn, const int32_t** ids_dev, const 
  * (gate then up), pairs f16 [tokens, k, H]. */
 int mfq_amd_moe_ffn_buffers(mfq_amd_moe_ffn* ffn, const void** gate_up_f16, const void** pairs_f16);
 /* Packed-weight bytes (all packed fields of every distinct routed expert, codebooks excluded) that
- * the last run's routing touched; synchronises the stream it ran on. */
+ * the last run's routing touched.  A measurement aid: runs a small kernel over the ids of the last run (which
+ * must still be valid) on the stream it ran on, and synchronises that stream. */
 int mfq_amd_moe_ffn_touched_bytes(mfq_amd_moe_ffn* ffn, int64_t* bytes, int32_t* distinct_experts);
 /* Measurement aid: when enabled, run() records HIP events on its stream around the five stages
  * (route plan, gate+up, SwiGLU, down, reduce) without synchronising; stage_times() synchronises the

@@ -519,6 +519,7 @@ struct mfq_amd_moe_ffn {
     PlanItem* d_item_info = nullptr;
     PairItem* d_pair_items = nullptr;
     ExpertInfo* d_expert_info = nullptr;
+    uint32_t* d_expert_words = nullptr;
     int32_t *d_expert_pool = nullptr, *d_items = nullptr, *d_class_offsets = nullptr, *d_tile_items = nullptr,
             *d_tile_offsets = nullptr, *d_counts = nullptr, *d_bounds = nullptr, *d_tile_bounds = nullptr,
             *d_tile_experts = nullptr, *d_ids_dst = nullptr, *d_distinct = nullptr;
@@ -533,12 +534,14 @@ struct mfq_amd_moe_ffn {
     uint32_t x_tile_layouts = 0;         // mask of those layouts   // decode only: activations as the streaming kernels read them
     int tile_capacity = 0;
     hipStream_t last_stream = nullptr;
+    const int32_t* last_ids = nullptr;   // routing of the last run (for touched_bytes)
+    int last_pairs = 0;
     bool decode_needs_items = true;   // some decode work runs on the exact kernels, which read the item lists
     bool timing = false;
     hipEvent_t events[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
 
     ~mfq_amd_moe_ffn() {
-        void* all[] = {d_pools, d_pool_class, d_pool_bytes, d_expert_pool, d_expert_info, d_item_info, d_pair_items, d_items, d_class_offsets, d_tile_items,
+        void* all[] = {d_pools, d_pool_class, d_pool_bytes, d_expert_pool, d_expert_info, d_expert_words, d_item_info, d_pair_items, d_items, d_class_offsets, d_tile_items,
                        d_tile_offsets, d_counts, d_bounds, d_tile_bounds, d_tile_experts, d_ids_dst, d_distinct,
                        d_touched, d_gu, d_hidden, d_pairs, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base};
         for (void* p : all) if (p) (void)hipFree(p);
@@ -616,6 +619,11 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
             }
             f->d_expert_info = device_alloc<ExpertInfo>(info.size());
             MFQ_HIP(hipMemcpy(f->d_expert_info, info.data(), sizeof(ExpertInfo) * info.size(), hipMemcpyHostToDevice));
+            MFQ_REQUIRE(pools <= 64, "at most 64 pools per FFN");
+            std::vector<uint32_t> words(info.size());
+            for (size_t i = 0; i < info.size(); ++i) words[i] = expert_word(info[i].pool, info[i].local, info[i].cls);
+            f->d_expert_words = device_alloc<uint32_t>(words.size());
+            MFQ_HIP(hipMemcpy(f->d_expert_words, words.data(), sizeof(uint32_t) * words.size(), hipMemcpyHostToDevice));
         }
         f->d_items = device_alloc<int32_t>(kSlots * E);
         f->d_item_info = device_alloc<PlanItem>(kSlots * E);
@@ -671,6 +679,8 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
              void* out_dev, hipStream_t stream, const PlanRoute* route) {
     {
         f->last_stream = stream;
+        f->last_ids = ids_dev;
+        f->last_pairs = tokens * f->top_k;
         const int E = f->experts, k = f->top_k, H = f->hidden, I = f->intermediate;
         const int pairs = tokens * k;
         const bool decode = tokens <= f->decode_limit;
@@ -686,14 +696,16 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         x.pools = f->d_pools; x.pool_class = f->d_pool_class; x.pool_bytes = f->d_pool_bytes;
         for (int s = 0; s <= kSlots; ++s) x.slot_pool_begin[s] = f->tables.slot_begin[s];
         x.slots = kSlots;
-        x.expert_pool = nullptr; x.expert_info = f->d_expert_info;
+        x.expert_pool = nullptr; x.expert_info = f->d_expert_info; x.expert_words = f->d_expert_words;
         x.items = f->d_items; x.item_info = f->d_item_info; x.pair_items = decode ? f->d_pair_items : nullptr; x.class_offsets = f->d_class_offsets;
         x.tile_items = f->d_tile_items; x.tile_offsets = f->d_tile_offsets;
         x.touched_bytes = f->d_touched; x.distinct = f->d_distinct;
         x.tile_capacity = f->tile_capacity; x.prefill_tile_m = kPrefillTileM; x.want_tiles = decode ? 0 : 1;
         x.want_items = !decode || f->decode_needs_items;
         // up to four tokens: experts rarely repeat, so nothing is gained by sorting the pairs by expert
-        x.direct_pairs = decode && tokens <= 4 && !x.want_items && f->d_expert_info != nullptr && f->config.launch_mode == 0;
+        // a streaming decode step needs nothing but the pair lists
+        x.pairs_only = decode && !x.want_items && f->config.launch_mode == 0 && pairs <= kPlanSortPairs;
+        x.direct_pairs = !x.pairs_only && decode && tokens <= 4 && !x.want_items && f->d_expert_info != nullptr && f->config.launch_mode == 0;
         const bool fast_mode = decode && f->config.launch_mode == 0;
         const bool pack_x = fast_mode && f->d_x_packed != nullptr;
         const bool pack_hidden = fast_mode && f->d_hidden_packed != nullptr;
@@ -890,6 +902,9 @@ extern "C" int mfq_amd_moe_ffn_buffers(mfq_amd_moe_ffn* f, const void** gate_up_
 extern "C" int mfq_amd_moe_ffn_touched_bytes(mfq_amd_moe_ffn* f, int64_t* bytes, int32_t* distinct_experts) {
     return guarded([&] {
         MFQ_REQUIRE(f, "null argument");
+        MFQ_REQUIRE(f->last_ids != nullptr, "no run yet");
+        launch_touched_bytes(f->last_ids, f->last_pairs, f->experts, kSlots, f->d_expert_info, f->d_touched, f->d_distinct,
+                             f->last_stream);
         MFQ_HIP(hipStreamSynchronize(f->last_stream));
         if (bytes) MFQ_HIP(hipMemcpy(bytes, f->d_touched, sizeof(int64_t), hipMemcpyDeviceToHost));
         if (distinct_experts) MFQ_HIP(hipMemcpy(distinct_experts, f->d_distinct, sizeof(int32_t), hipMemcpyDeviceToHost));

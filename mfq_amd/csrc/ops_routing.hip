@@ -76,97 +76,202 @@ __device__ __forceinline__ long long dpp64(long long v) {
 }
 __device__ __forceinline__ long long max64(long long a, long long b) { return a > b ? a : b; }
 
+// LDS scratch of one 32-lane group of topk_token.
+constexpr int kTopkCandidates = 64;
+struct TopkScratch {
+    unsigned long long candidates[kTopkCandidates];   // (probability bits << 32) | ~expert: larger wins
+    int lane_best[32];                                // the best key of every lane
+    int selected[32];                                 // probability bits of rank r
+    int threshold;                                    // top_k-th largest of lane_best
+    int count;                                        // candidates found
+};
+
 // One 32-lane group per token, laid out like the reference kernels (lane owns experts lane,
 // lane+32, ...) so that the softmax denominator is summed in the same order
 // (mfq/kernels/cuda/moe.cu:1383-1446).  Selection works on integer keys: the bits of a non-negative
-// probability order like the value, a consumed or absent entry is -1, and ties go to the lower
-// expert id.  A lane keeps the best of its own entries; every rank takes the best of the 32 lane
-// candidates with lane-exchange steps, and only the winning lane rescans its entries.
-// Runs on the 32 lanes that share threadIdx.x / 32; `local_ids`, when given, also receives the ids
-// (any address space, e.g. LDS).
+// probability order like the value, an absent entry is -1, and ties go to the lower expert id.
+//
+// The top_k-th largest of the 32 per-lane maxima is a lower bound of the top_k-th largest entry (at least top_k
+// entries reach it), so only entries at or above it can be selected: usually one or two dozen.  They are
+// collected in LDS and every one counts the candidates that beat it; its rank is that count.  When more than
+// kTopkCandidates entries reach the bound (many equal probabilities, or the large ones crowded into few lanes) the
+// group falls back to one selection round per rank: the best of the 32 lane candidates by lane exchanges, and the
+// winning lane rescans its entries.  Both give the same ids: the order (probability, then lower id) is total.
+//
+// Every thread of the block calls it (block-wide barriers inside); groups with active == false select nothing.
+// `local_ids`, when given, also receives the ids (any address space, e.g. LDS).
 template <int SLOTS>
-__device__ __forceinline__ void topk_token(const void* logits, int dtype, int token, int experts, int top_k,
+__device__ __forceinline__ void topk_token(const void* logits, int dtype, int token, bool active, int experts, int top_k,
                                            int normalize, float norm_floor, float scale, int32_t* ids,
-                                           float* weights, int* local_ids) {
+                                           float* weights, int* local_ids, TopkScratch* scratch) {
     const int lane = threadIdx.x & 31;
-    const int64_t base = static_cast<int64_t>(token) * experts;
-    // all loads of the lane are issued before the first value is looked at: the type switch sits
-    // outside the loops and absent entries read a valid address
+    const bool busy = __ballot(active) != 0ull;          // waves without a token only keep the barriers
     float cached[SLOTS];
-    if (dtype == MFQ_AMD_F32) {
-        const float* p = static_cast<const float*>(logits) + base;
+    float total = 1.0f;
+    int lane_best = -1;
+    if (busy) {
+        const int64_t base = static_cast<int64_t>(active ? token : 0) * experts;
+        // all loads of the lane are issued before the first value is looked at: the type switch sits
+        // outside the loops and absent entries read a valid address
+        if (dtype == MFQ_AMD_F32) {
+            const float* p = static_cast<const float*>(logits) + base;
 #pragma unroll
-        for (int slot = 0; slot < SLOTS; ++slot) cached[slot] = p[lane + slot * 32 < experts ? lane + slot * 32 : 0];
-    } else {
-        const uint16_t* p = static_cast<const uint16_t*>(logits) + base;
-        uint16_t raw[SLOTS];
+            for (int slot = 0; slot < SLOTS; ++slot) cached[slot] = p[lane + slot * 32 < experts ? lane + slot * 32 : 0];
+        } else {
+            const uint16_t* p = static_cast<const uint16_t*>(logits) + base;
+            uint16_t raw[SLOTS];
 #pragma unroll
-        for (int slot = 0; slot < SLOTS; ++slot) raw[slot] = p[lane + slot * 32 < experts ? lane + slot * 32 : 0];
-#pragma unroll
-        for (int slot = 0; slot < SLOTS; ++slot)
-            cached[slot] = dtype == MFQ_AMD_F16 ? half_bits_to_float(raw[slot]) : bf16_bits_to_float(raw[slot]);
-    }
-    float maximum = -__builtin_inff();
-#pragma unroll
-    for (int slot = 0; slot < SLOTS; ++slot) {
-        const float v = cached[slot];
-        cached[slot] = lane + slot * 32 >= experts ? -__builtin_inff() : v != v ? -3.402823466e+38f : v;
-        maximum = fmaxf(maximum, cached[slot]);
-    }
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset, 32));
-    float sum = 0.0f;
-#pragma unroll
-    for (int slot = 0; slot < SLOTS; ++slot) {
-        if (lane + slot * 32 < experts) {
-            cached[slot] = routing_expf(cached[slot] - maximum);
-            sum = sum + cached[slot];
-        }
-    }
-    const float total = tree32_sum(sum);
-    int key[SLOTS];
-#pragma unroll
-    for (int slot = 0; slot < SLOTS; ++slot)
-        key[slot] = lane + slot * 32 < experts ? static_cast<int>(__float_as_uint(cached[slot] / total)) : -1;
-
-    auto local_best = [&](int& best, int& best_slot) {
-        best = -1; best_slot = 0;
-#pragma unroll
-        for (int slot = 0; slot < SLOTS; ++slot)
-            if (key[slot] > best) { best = key[slot]; best_slot = slot; }
-    };
-    int best, best_slot;
-    local_best(best, best_slot);
-
-    float selected = 0.0f;
-    for (int rank = 0; rank < top_k; ++rank) {
-        // candidate of this lane: (probability bits, ~expert); larger wins
-        long long candidate = (static_cast<long long>(best) << 32) | static_cast<uint32_t>(~(lane + 32 * best_slot));
-        candidate = max64(candidate, dpp64<0xB1>(candidate));    // lane ^ 1
-        candidate = max64(candidate, dpp64<0x4E>(candidate));    // lane ^ 2
-        candidate = max64(candidate, dpp64<0x141>(candidate));   // mirror inside 8 lanes
-        candidate = max64(candidate, dpp64<0x140>(candidate));   // mirror inside 16 lanes
-        candidate = max64(candidate, __shfl_xor(candidate, 16, 32));
-        const int expert = static_cast<int>(~static_cast<uint32_t>(candidate));
-        const int bits = static_cast<int>(candidate >> 32);
-        if (lane == rank) {
-            selected = __uint_as_float(static_cast<uint32_t>(bits));
-            ids[static_cast<int64_t>(token) * top_k + rank] = expert;
-            if (local_ids != nullptr) local_ids[token * top_k + rank] = expert;
-        }
-        if (lane == (expert & 31)) {
-            const int taken = expert >> 5;
+            for (int slot = 0; slot < SLOTS; ++slot) raw[slot] = p[lane + slot * 32 < experts ? lane + slot * 32 : 0];
 #pragma unroll
             for (int slot = 0; slot < SLOTS; ++slot)
-                if (slot == taken) key[slot] = -1;
-            local_best(best, best_slot);
+                cached[slot] = dtype == MFQ_AMD_F16 ? half_bits_to_float(raw[slot]) : bf16_bits_to_float(raw[slot]);
+        }
+        float maximum = -__builtin_inff();
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) {
+            const float v = cached[slot];
+            cached[slot] = lane + slot * 32 >= experts ? -__builtin_inff() : v != v ? -3.402823466e+38f : v;
+            maximum = fmaxf(maximum, cached[slot]);
+        }
+#pragma unroll
+        for (int offset = 16; offset > 0; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset, 32));
+        float sum = 0.0f;
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) {
+            if (lane + slot * 32 < experts) {
+                cached[slot] = routing_expf(cached[slot] - maximum);
+                sum = sum + cached[slot];
+            } else {
+                cached[slot] = -1.0f;                     // absent: the bits of a negative number are a negative key
+            }
+        }
+        total = tree32_sum(sum);
+        // The numerators order like the probabilities (division by the common total is monotone), except that
+        // numerators a few units in the last place apart may give the same probability: the bound below is taken
+        // on the numerators and lowered by that much, the probabilities themselves are computed for candidates only.
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) {
+            const int bits = active ? static_cast<int>(__float_as_uint(cached[slot])) : -1;
+            lane_best = bits > lane_best ? bits : lane_best;
+        }
+        scratch->lane_best[lane] = lane_best;
+        if (lane == 0) { scratch->threshold = 0x7fffffff; scratch->count = 0; }
+    }
+    __syncthreads();
+    if (busy) {
+        // the top_k-th largest lane maximum: the smallest one that fewer than top_k others exceed
+        int greater = 0;
+#pragma unroll
+        for (int i = 0; i < 32; i += 4) {
+            const int4 v = *reinterpret_cast<const int4*>(&scratch->lane_best[i]);
+            greater += (v.x > lane_best) + (v.y > lane_best) + (v.z > lane_best) + (v.w > lane_best);
+        }
+        if (greater < top_k) atomicMin(&scratch->threshold, lane_best);
+    }
+    __syncthreads();
+    if (busy) {
+        const int bound = scratch->threshold - 8 > 0 ? scratch->threshold - 8 : 0;
+        int mine = 0;
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) mine += active && static_cast<int>(__float_as_uint(cached[slot])) >= bound;
+        int at = mine > 0 ? atomicAdd(&scratch->count, mine) : 0;
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) {
+            const uint32_t bits = __float_as_uint(cached[slot]);
+            if (active && static_cast<int>(bits) >= bound) {
+                if (at < kTopkCandidates)
+                    scratch->candidates[at] = (static_cast<unsigned long long>(bits) << 32) | static_cast<uint32_t>(~(lane + 32 * slot));
+                ++at;
+            }
         }
     }
-    float denominator = 1.0f;
-    if (normalize) denominator = fmaxf(tree32_sum(lane < top_k ? selected : 0.0f), norm_floor);
-    if (lane < top_k) {
-        const float value = normalize ? selected / denominator : selected;
-        weights[static_cast<int64_t>(token) * top_k + lane] = value * scale;
+    __syncthreads();
+    const int found = busy ? scratch->count : 0;
+    // (numerators below 2^-100 can give subnormal probabilities, where many more numerators share one quotient)
+    const bool by_rounds = active && (found > kTopkCandidates || found < top_k || scratch->threshold < 0x0D800000);
+    unsigned long long mine2[kTopkCandidates / 32];
+    if (busy && active && !by_rounds) {
+        // numerator -> probability, for the candidates only
+#pragma unroll
+        for (int j = 0; j < kTopkCandidates / 32; ++j) {
+            const int at = lane + 32 * j;
+            mine2[j] = 0ull;
+            if (at < found) {
+                const unsigned long long c = scratch->candidates[at];
+                const float probability = __uint_as_float(static_cast<uint32_t>(c >> 32)) / total;
+                mine2[j] = (static_cast<unsigned long long>(__float_as_uint(probability)) << 32) | (c & 0xffffffffull);
+            }
+        }
+    }
+    __syncthreads();
+    if (busy && active && !by_rounds) {
+#pragma unroll
+        for (int j = 0; j < kTopkCandidates / 32; ++j)
+            if (lane + 32 * j < found) scratch->candidates[lane + 32 * j] = mine2[j];
+    }
+    __syncthreads();
+    if (busy && active && !by_rounds) {
+#pragma unroll
+        for (int j = 0; j < kTopkCandidates / 32; ++j) {
+            if (lane + 32 * j >= found) continue;
+            const unsigned long long me = mine2[j];
+            int rank = 0;
+            for (int i = 0; i < found; ++i) rank += scratch->candidates[i] > me;
+            if (rank < top_k) {
+                const int expert = static_cast<int>(~static_cast<uint32_t>(me));
+                ids[static_cast<int64_t>(token) * top_k + rank] = expert;
+                if (local_ids != nullptr) local_ids[token * top_k + rank] = expert;
+                scratch->selected[rank] = static_cast<int>(me >> 32);
+            }
+        }
+    }
+    if (by_rounds) {
+        // one selection round per rank on the probabilities of every entry
+        int key[SLOTS];
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot)
+            key[slot] = lane + slot * 32 < experts ? static_cast<int>(__float_as_uint(cached[slot] / total)) : -1;
+        auto local_best = [&](int& best, int& best_slot) {
+            best = -1; best_slot = 0;
+#pragma unroll
+            for (int slot = 0; slot < SLOTS; ++slot)
+                if (key[slot] > best) { best = key[slot]; best_slot = slot; }
+        };
+        int best, best_slot;
+        local_best(best, best_slot);
+        for (int rank = 0; rank < top_k; ++rank) {
+            // candidate of this lane: (probability bits, ~expert); larger wins
+            long long candidate = (static_cast<long long>(best) << 32) | static_cast<uint32_t>(~(lane + 32 * best_slot));
+            candidate = max64(candidate, dpp64<0xB1>(candidate));    // lane ^ 1
+            candidate = max64(candidate, dpp64<0x4E>(candidate));    // lane ^ 2
+            candidate = max64(candidate, dpp64<0x141>(candidate));   // mirror inside 8 lanes
+            candidate = max64(candidate, dpp64<0x140>(candidate));   // mirror inside 16 lanes
+            candidate = max64(candidate, __shfl_xor(candidate, 16, 32));
+            const int expert = static_cast<int>(~static_cast<uint32_t>(candidate));
+            const int bits = static_cast<int>(candidate >> 32);
+            if (lane == rank) {
+                scratch->selected[rank] = bits;
+                ids[static_cast<int64_t>(token) * top_k + rank] = expert;
+                if (local_ids != nullptr) local_ids[token * top_k + rank] = expert;
+            }
+            if (lane == (expert & 31)) {
+                const int taken = expert >> 5;
+#pragma unroll
+                for (int slot = 0; slot < SLOTS; ++slot)
+                    if (slot == taken) key[slot] = -1;
+                local_best(best, best_slot);
+            }
+        }
+    }
+    __syncthreads();
+    if (busy) {
+        const float selected = active && lane < top_k ? __uint_as_float(static_cast<uint32_t>(scratch->selected[lane])) : 0.0f;
+        float denominator = 1.0f;
+        if (normalize) denominator = fmaxf(tree32_sum(selected), norm_floor);
+        if (active && lane < top_k) {
+            const float value = normalize ? selected / denominator : selected;
+            weights[static_cast<int64_t>(token) * top_k + lane] = value * scale;
+        }
     }
 }
 
@@ -174,9 +279,10 @@ template <int SLOTS>
 __global__ void __launch_bounds__(64) topk_kernel(const void* logits, int dtype, int tokens, int experts,
                                                   int top_k, int normalize, float norm_floor, float scale,
                                                   int32_t* ids, float* weights) {
+    __shared__ TopkScratch scratch[2];
     const int token = blockIdx.x * 2 + (threadIdx.x >> 5);
-    if (token >= tokens) return;
-    topk_token<SLOTS>(logits, dtype, token, experts, top_k, normalize, norm_floor, scale, ids, weights, nullptr);
+    topk_token<SLOTS>(logits, dtype, token, token < tokens, experts, top_k, normalize, norm_floor, scale, ids, weights, nullptr,
+                      &scratch[threadIdx.x >> 5]);
 }
 
 // -------------------------------------------------------- route plan ----
@@ -480,6 +586,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_small_kernel(PlanArgs
     __shared__ unsigned long long group_counts[kSlots][kPlanThreads / 64];  // per wave of positions: pairs per cost group
     __shared__ unsigned long long total_bytes;
     __shared__ int total_distinct, repeated;
+    __shared__ TopkScratch topk_scratch[TOPK_SLOTS > 0 ? kPlanThreads / 32 : 1];
     if (blockIdx.x > 0) {
         const int row = blockIdx.x - 1;
         const int element = a.pack.dtype == MFQ_AMD_F32 ? 4 : 2;
@@ -504,10 +611,9 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_small_kernel(PlanArgs
         expert_of[tid] = -1;
         __syncthreads();
         const int token = tid >> 5;
-        if (token < a.route.tokens)
-            topk_token<(TOPK_SLOTS > 0 ? TOPK_SLOTS : 1)>(a.route.logits, a.route.dtype, token, E, a.top_k, a.route.normalize,
-                                                          a.route.norm_floor, a.route.scale, a.route.ids_out,
-                                                          a.route.weights_out, expert_of);
+        topk_token<(TOPK_SLOTS > 0 ? TOPK_SLOTS : 1)>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
+                                                      a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
+                                                      a.route.weights_out, expert_of, &topk_scratch[token]);
         __syncthreads();
         expert = expert_of[tid];
     } else {
@@ -724,7 +830,133 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_small_kernel(PlanArgs
     if (tid == 0) { *x.touched_bytes = static_cast<int64_t>(total_bytes); *x.distinct = total_distinct; }
 }
 
+// The plan of a streaming decode step: nothing but the per-slot pair lists, costliest group first and inside a
+// group by expert (pairs of one expert adjacent, so its weights leave HBM once), then by pair.  That order is a
+// total order on a 23-bit key per (slot, pair), so a pair's position is the number of smaller keys: every
+// (slot, pair) counts them against the keys in LDS, split over `parts` neighbouring lanes when threads are to spare.
+// No histograms, scans or per-expert lists; one barrier after the keys are written.
+// TOPK_SLOTS > 0: the ids are selected here first from router logits, as in route_plan_small_kernel.
+template <int TOPK_SLOTS>
+__global__ void __launch_bounds__(kPlanThreads) route_plan_pairs_kernel(PlanArgs a) {
+    __shared__ __align__(16) uint32_t keys[kSlots][kPlanSortPairs];
+    __shared__ __align__(16) int4 records[kSlots][kPlanSortPairs];      // PairItem of (slot, pair)
+    __shared__ int expert_of[kPlanThreads];
+    __shared__ uint32_t expert_words[kSlots][kPlanMaxExperts];
+    __shared__ float pack_scratch[kPlanThreads / 64];
+    __shared__ TopkScratch topk_scratch[TOPK_SLOTS > 0 ? kPlanThreads / 32 : 1];
+    if (blockIdx.x > 0) {
+        const int row = blockIdx.x - 1;
+        const int element = a.pack.dtype == MFQ_AMD_F32 ? 4 : 2;
+        xpack_row(static_cast<const char*>(a.pack.src) + static_cast<int64_t>(row) * a.pack.width * element, a.pack.dtype,
+                  a.pack.vector_ok != 0, a.pack.width, a.pack.dst + row * a.pack.stride, pack_scratch);
+        return;
+    }
+    const int E = a.experts, P = a.pairs;
+    const int tid = threadIdx.x;
+    const PlanExtras& x = a.extras;
+    // the per-expert records of every slot, requested first and parked in LDS once the routes are known
+    uint32_t words[kSlots];
+#pragma unroll
+    for (int s = 0; s < kSlots; ++s) words[s] = s < x.slots && tid < E ? x.expert_words[s * E + tid] : kExpertAbsent;
+    if (TOPK_SLOTS > 0) {
+        const int token = tid >> 5;
+        topk_token<(TOPK_SLOTS > 0 ? TOPK_SLOTS : 1)>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
+                                                      a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
+                                                      a.route.weights_out, expert_of, &topk_scratch[token]);
+    } else if (tid < P) {
+        expert_of[tid] = a.ids[tid];
+    }
+#pragma unroll
+    for (int s = 0; s < kSlots; ++s) expert_words[s][tid] = words[s];
+    __syncthreads();
+    // keys and records of every (slot, pair)
+    const int items = x.slots * P;
+    for (int item = tid; item < items; item += kPlanThreads) {
+        const int s = item / P, p = item - s * P;
+        const int expert = expert_of[p];
+        int4 record = {-1, 0, 0, -1};
+        int group = 7;                                    // unrouted pairs and experts without a pool: behind everything
+        if (static_cast<unsigned>(expert) < static_cast<unsigned>(E)) {
+            const uint32_t word = expert_words[s][expert];
+            if (word != kExpertAbsent) {
+                const int cls = static_cast<int>(word & 0x1ffu);
+                record = int4{p, static_cast<int>((word >> 9) & 0x3fu), static_cast<int>((word >> 15) & 0x3ffu), cls};
+                group = cost_group(cls);
+            }
+        }
+        records[s][p] = record;
+        keys[s][p] = (static_cast<uint32_t>(group) << 20) | (static_cast<uint32_t>(record.x >= 0 ? expert : 0) << 10) |
+                     static_cast<uint32_t>(p);
+    }
+    // keys behind the last pair compare larger than any real one, so that whole vectors can be scanned
+    for (int i = tid; i < kSlots * 4; i += kPlanThreads)
+        if (P + (i & 3) < kPlanSortPairs) keys[i >> 2][P + (i & 3)] = 0xffffffffu;
+    __syncthreads();
+    int parts = 1;
+    while (parts < 8 && items * parts * 2 <= kPlanThreads) parts *= 2;
+    const int chunk = ((P + parts - 1) / parts + 3) & ~3;     // keys per part, a multiple of four
+    const int rounds = (items * parts + kPlanThreads - 1) / kPlanThreads;
+    for (int round = 0; round < rounds; ++round) {
+        const int index = round * kPlanThreads + tid;
+        const int item = index / parts, part = index - item * parts;
+        const bool live = item < items;
+        const int s = live ? item / P : 0, p = live ? item - s * P : 0;
+        const uint32_t mine = keys[s][p];
+        int smaller = 0;
+        const int begin = part * chunk, end = begin + chunk < P ? begin + chunk : P;
+        for (int q = begin; q < end; q += 4) {
+            const uint4 v = *reinterpret_cast<const uint4*>(&keys[s][q]);
+            smaller += (v.x < mine) + (v.y < mine) + (v.z < mine) + (v.w < mine);
+        }
+        // the parts of an item sit in neighbouring lanes
+        for (int step = 1; step < parts; step *= 2) smaller += __shfl_xor(smaller, step, 64);
+        if (live && part == 0) {
+            const int4 record = records[s][p];
+            x.pair_items[static_cast<int64_t>(s) * P + smaller] = PairItem{record.x, record.y, record.z, record.w};
+        }
+    }
+}
+
+// Packed bytes and distinct experts of a routing: a measurement aid, off the step's path.
+__global__ void __launch_bounds__(kPlanThreads) touched_bytes_kernel(const int32_t* ids, int pairs, int experts, int slots,
+                                                                     const ExpertInfo* expert_info, int64_t* touched_bytes,
+                                                                     int32_t* distinct) {
+    __shared__ int seen[kPlanMaxExperts];
+    __shared__ unsigned long long total_bytes;
+    __shared__ int total_distinct;
+    const int tid = threadIdx.x;
+    if (tid < experts) seen[tid] = 0;
+    if (tid == 0) { total_bytes = 0ull; total_distinct = 0; }
+    __syncthreads();
+    for (int p = tid; p < pairs; p += kPlanThreads) {
+        const int e = ids[p];
+        if (static_cast<unsigned>(e) < static_cast<unsigned>(experts)) seen[e] = 1;
+    }
+    __syncthreads();
+    if (tid < experts && seen[tid]) {
+        unsigned long long bytes = 0ull;
+        bool any = false;
+        for (int s = 0; s < slots; ++s) {
+            const ExpertInfo info = expert_info[s * experts + tid];
+            if (info.pool >= 0) { bytes += static_cast<unsigned long long>(info.bytes); any = true; }
+        }
+        atomicAdd(&total_bytes, bytes);
+        (void)any;
+        atomicAdd(&total_distinct, 1);
+    }
+    __syncthreads();
+    if (tid == 0) { *touched_bytes = static_cast<int64_t>(total_bytes); *distinct = total_distinct; }
+}
+
 }  // namespace dev
+
+void launch_touched_bytes(const int32_t* ids, int pairs, int experts, int slots, const ExpertInfo* expert_info,
+                          int64_t* touched_bytes, int32_t* distinct, hipStream_t stream) {
+    MFQ_REQUIRE(experts > 0 && experts <= kPlanMaxExperts && pairs >= 0, "invalid routing geometry");
+    hipLaunchKernelGGL(dev::touched_bytes_kernel, dim3(1), dim3(kPlanThreads), 0, stream, ids, pairs, experts, slots, expert_info,
+                       touched_bytes, distinct);
+    check_launch("touched_bytes_kernel");
+}
 
 void raise_routing_limits() {
     MFQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::route_plan_kernel),
@@ -747,6 +979,26 @@ void launch_route_plan(const PlanArgs& args, hipStream_t stream) {
                     (args.pairs <= kPlanThreads && args.extras.items != nullptr && args.extras.expert_info != nullptr &&
                      args.extras.pair_items != nullptr && !args.extras.want_tiles && !args.extras.want_items),
                 "pair records in pair order need a decode-sized plan with resolved expert records and no other lists");
+    if (args.extras.pairs_only) {
+        MFQ_REQUIRE(args.pairs <= kPlanSortPairs && args.extras.expert_words != nullptr && args.extras.pair_items != nullptr &&
+                        !args.extras.want_tiles && !args.extras.want_items && args.extras.slots >= 1 && args.extras.slots <= kSlots,
+                    "the pairs-only plan needs resolved expert records and at most 512 pairs");
+        const dim3 grid(1 + pack_rows);
+        auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(kPlanThreads), 0, stream, args); };
+        if (args.route.logits == nullptr) {
+            launch(dev::route_plan_pairs_kernel<0>);
+        } else {
+            MFQ_REQUIRE(args.route.tokens <= kPlanThreads / 32 && args.route.tokens * args.top_k == args.pairs &&
+                        args.top_k >= 1 && args.top_k <= 32 && args.top_k <= args.experts,
+                        "fused routing serves at most 32 tokens");
+            if (args.experts <= 128) launch(dev::route_plan_pairs_kernel<4>);
+            else if (args.experts <= 256) launch(dev::route_plan_pairs_kernel<8>);
+            else if (args.experts <= 512) launch(dev::route_plan_pairs_kernel<16>);
+            else launch(dev::route_plan_pairs_kernel<32>);
+        }
+        check_launch("route_plan_pairs_kernel");
+        return;
+    }
     if (args.pairs <= kPlanThreads && (args.extras.items == nullptr || !args.extras.want_tiles)) {
         const dim3 grid(1 + pack_rows);
         auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(kPlanThreads), 0, stream, args); };

@@ -45,6 +45,13 @@ struct ExpertInfo {
     int64_t bytes;    // packed bytes of the expert
 };
 
+// An ExpertInfo in one word: class word (9 bits) | pool << 9 (6 bits) | local << 15 (10 bits); all ones = absent.
+constexpr uint32_t kExpertAbsent = 0xffffffffu;
+inline uint32_t expert_word(int pool, int local, int cls_word) {
+    return pool < 0 ? kExpertAbsent
+                    : static_cast<uint32_t>(cls_word & 0x1ff) | (static_cast<uint32_t>(pool) << 9) | (static_cast<uint32_t>(local) << 15);
+}
+
 // Work lists the routed-projection kernels consume, all in device memory.
 //   expert_pool[s][e]   index (into pools) of the pool that holds expert e in slot s, -1 = absent
 //   items[s][i]         active experts of slot s sorted by (kernel class, expert id)
@@ -60,6 +67,7 @@ struct PlanExtras {
     int32_t slots;                     // 1..3
     int32_t* expert_pool;              // [slots][experts], written unless expert_info is given
     const ExpertInfo* expert_info;     // [slots][experts] precomputed (pools never change between runs), or null
+    const uint32_t* expert_words;      // [slots][experts] the same records in one word each (expert_word()), for pairs_only
     int32_t* items;                    // [slots][experts]
     PlanItem* item_info;               // [slots][experts] same order as items
     PairItem* pair_items;              // [slots][pairs]
@@ -75,7 +83,11 @@ struct PlanExtras {
     int32_t direct_pairs;              // 1 (decode-sized plans with expert_info and without want_items / want_tiles only):
                                        // pair_items in pair order, nothing sorted, and none of counts, expert_bounds,
                                        // ids_dst, items written; for batches so small that experts rarely repeat
+    int32_t pairs_only;                // 1 (at most kPlanSortPairs pairs, expert_info given, no want_items / want_tiles):
+                                       // only pair_items is produced, by the kernel that ranks the pairs directly;
+                                       // none of counts, expert_bounds, ids_dst, items, touched_bytes, distinct written
 };
+constexpr int kPlanSortPairs = 512;
 
 // Activation rows to bring into the packed form of the streaming kernels: one extra block per row.
 struct PlanPack {
@@ -111,5 +123,8 @@ struct PlanArgs {
 };
 
 void launch_route_plan(const PlanArgs& args, hipStream_t stream);
+// touched_bytes[0] = packed bytes of the distinct experts `ids` names over the slots of expert_info; distinct[0] = their number.
+void launch_touched_bytes(const int32_t* ids, int pairs, int experts, int slots, const ExpertInfo* expert_info,
+                          int64_t* touched_bytes, int32_t* distinct, hipStream_t stream);
 
 }  // namespace mfq_amd

@@ -102,3 +102,51 @@ def test_route_plan_skips_invalid_ids():
     ref = O.route_plan(ids, 8, 8)
     assert np.array_equal(plan["counts"].cpu().numpy(), ref["counts"])
     assert np.array_equal(plan["ids_dst"].cpu().numpy()[: ref["ids_dst"].size], ref["ids_dst"])
+
+
+def _check_topk(logits, k, **kwargs):
+    import torch
+    from mfq_amd import runtime as R
+    ids_ref, w_ref = O.topk(logits, k, **kwargs)
+    ids, w = R.moe_topk(torch.from_numpy(logits).cuda(), k, **kwargs)
+    assert np.array_equal(ids.cpu().numpy(), ids_ref)
+    np.testing.assert_allclose(w.cpu().numpy(), w_ref, rtol=1e-6, atol=1e-38)
+
+
+def test_topk_adversarial_layouts():
+    """Inputs chosen against the selection's shortcuts: more equal maxima than routes; the large logits crowded into
+    one lane's entries (experts 3, 35, 67, ...); logits one unit in the last place apart (numerators that may share a
+    probability); a one-hot row (probabilities near the bottom of the range); coarse logits with many exact ties."""
+    rng = np.random.default_rng(123)
+    rows = []
+    a = rng.normal(0, 1, 512).astype(np.float32); a[[5, 37, 69, 100, 101, 200, 300, 301, 302, 400, 450, 511]] = 4.0
+    rows.append(a)                                                      # 12 equal maxima, top-10
+    b = rng.normal(0, 1, 512).astype(np.float32); b[3::32] = 3.0 + np.arange(16, dtype=np.float32) * 0.125
+    rows.append(b)                                                      # the 16 largest in the entries of lane 3
+    c = np.float32(1.0) + np.arange(512, dtype=np.float32) * np.float32(2.0 ** -23)
+    rows.append(c[::-1].copy())                                         # neighbours one ulp apart, descending by id
+    rows.append(c.copy())
+    d = np.zeros(512, dtype=np.float32); d[77] = 100.0
+    rows.append(d)                                                      # one-hot: the rest underflows to equal tiny values
+    e = np.zeros(512, dtype=np.float32); e[77] = 60.0; e[100:140] = rng.normal(0, 0.001, 40)
+    rows.append(e)
+    rows.append(np.round(rng.normal(0, 1, 512) * 4).astype(np.float32) / 4)     # quantised: many exact ties
+    rows.append(np.round(rng.normal(0, 1, 512) * 2).astype(np.float32) / 2)
+    rows.append(np.full(512, -1e30, dtype=np.float32))
+    f = rng.normal(0, 1, 512).astype(np.float32); f[::3] = np.nan
+    rows.append(f)
+    logits = np.stack(rows)
+    for k in (1, 4, 10, 32):
+        _check_topk(logits, k)
+    _check_topk(logits, 10, normalize=False, scale=0.5)
+    for experts, k in ((40, 4), (33, 8), (64, 32), (1000, 10), (129, 6)):
+        sub = np.round(rng.normal(0, 1, (9, experts)) * 3).astype(np.float32) / 3
+        _check_topk(sub, k)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_topk_many_random_rows(seed):
+    rng = np.random.default_rng(1000 + seed)
+    logits = rng.normal(0, [0.02, 1.0, 8.0][seed], (257, 512)).astype(np.float32)
+    _check_topk(logits, 10)
+    _check_topk(logits[:33, :256].copy(), 8)
