@@ -227,7 +227,7 @@ __device__ __forceinline__ void pack_block(const float (&x)[32], float down, con
     _Float16 h[32];
 #pragma unroll
     for (int i = 0; i < 32; ++i) h[i] = static_cast<_Float16>(b.valid ? x[i] * down : 0.0f);
-    float plain[4] = {0.0f, 0.0f, 0.0f, 0.0f};   // per chunk
+    float plain[4] = {0.0f, 0.0f, 0.0f, 0.0f};   // per chunk, columns added in ascending order (as xpack_row does)
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
         const int first = pair_column<CLS>(k, 0), second = pair_column<CLS>(k, 1);
@@ -235,10 +235,9 @@ __device__ __forceinline__ void pack_block(const float (&x)[32], float down, con
         pair[0] = static_cast<_Float16>(static_cast<float>(h[first]) * pair_scale<CLS>(k));
         pair[1] = static_cast<_Float16>(static_cast<float>(h[second]) * pair_scale<CLS>(k));
         out.p[k] = __builtin_bit_cast(uint32_t, pair);
-        // both columns of a pair lie in the same quantisation group
-        const float sum = static_cast<float>(h[first]) + static_cast<float>(h[second]);
-        plain[first / 8] += sum;
     }
+#pragma unroll
+    for (int i = 0; i < 32; ++i) plain[i / 8] += static_cast<float>(h[i]);
     out.g0 = out.g1 = 0.0f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {

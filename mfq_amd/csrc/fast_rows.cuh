@@ -21,11 +21,18 @@ struct XSource {
     const void* row;     // first element of the token's activation row, or of its packed form (xpack.cuh)
     int dtype;
     bool vector_ok;
+    const float* scale;  // kXScaled: {2^-e, 2^e} of the row, readable once the prologue has run
 };
+constexpr int kXRaw = 0, kXPacked = 1, kXScaled = 2;
+struct NoPrologue { __device__ __forceinline__ void operator()() const {} };
 
 // Rows [row_begin, row_end) of one expert times NT tokens.  LPR lanes share a row (64, or 16 when the
 // row has at most 512 columns and a wave covers four rows at a time); SLABS lane blocks per lane.
-// PACKED: the activation rows are in the packed form of xpack.cuh.
+// XMODE: where the activations come from.  kXRaw: rows of fp16 / bf16 values (global memory or LDS); the largest
+// magnitude is found here.  kXPacked: rows in the packed form of xpack.cuh.  kXScaled: rows of fp16 values whose
+// normaliser the caller already knows (XSource::scale_down / scale_up), e.g. values a block staged in LDS.
+// `prologue()` runs once, after the first loads of packed rows have been issued and before the activations are
+// read: block-wide work (it may contain barriers) that produces the activations overlaps those loads.
 // The packed data of RING row slots is in flight at any time: a slot's registers are refilled with
 // the slot RING places further on as soon as it has been consumed, so loads overlap the arithmetic
 // of the RING - 1 slots in between.  SLOTS > 0: the call covers exactly SLOTS row slots starting at
@@ -33,9 +40,9 @@ struct XSource {
 // sequence is straight-line code, which lets the compiler wait for exactly the loads a slot needs;
 // SLOTS == 0: any number of rows, looped.  store(n, row, value) is called by one lane per (token, row).
 // IB: index bits of the NVQ format when known at compile time (0: looked up per row).
-template <int CLS, int LPR, int SLABS, int NT, int RING, bool PACKED, int SLOTS, int IB = 0, class Store>
+template <int CLS, int LPR, int SLABS, int NT, int RING, int XMODE, int SLOTS, int IB = 0, class Store, class Prologue = NoPrologue>
 __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (&xs)[NT], int width, int row_begin,
-                                          int row_end, int out_rows, Store&& store) {
+                                          int row_end, int out_rows, Store&& store, Prologue&& prologue = Prologue()) {
     using C = FastClass<CLS>;
     constexpr int SUBS = kWave / LPR;          // rows per slot
     constexpr int R = RING < 4 ? RING : 4;     // slots whose totals are reduced together
@@ -79,12 +86,14 @@ __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (
         }
     }
 
+    prologue();
+
     // activations: already packed, or: load, find the largest magnitude of the token, normalise and pack
     XBlock x[SLABS][NT];
     float up[NT];
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
-        if constexpr (PACKED) {
+        if constexpr (XMODE == kXPacked) {
             const uint32_t* row = static_cast<const uint32_t*>(xs[n].row);
             up[n] = gload<float>(row + xpack_scale_at(width));
 #pragma unroll
@@ -100,9 +109,13 @@ __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (
 #pragma unroll
                 for (int i = 0; i < 32; ++i) largest = fmaxf(largest, blocks[s].valid ? fabsf(values[s][i]) : 0.0f);
             }
-            largest = wave_max(largest);
             float down;
-            normaliser(largest, down, up[n]);
+            if constexpr (XMODE == kXScaled) {
+                down = xs[n].scale[0]; up[n] = xs[n].scale[1];
+            } else {
+                largest = wave_max(largest);
+                normaliser(largest, down, up[n]);
+            }
 #pragma unroll
             for (int s = 0; s < SLABS; ++s) pack_block<CLS>(values[s], down, blocks[s], x[s][n]);
         }

@@ -32,6 +32,10 @@ struct RowsArgs {
     int64_t in_packed_stride;          // dwords between packed rows
     const uint16_t* in_tiles;          // the same rows as fp16 in the pair order of the weight classes (tile kernel), or null
     int64_t in_tiles_layout_stride;    // halves between the copies in the four pair layouts; 0: rows are in the order their consumer needs
+    const uint16_t* gu;                // streaming decode kernel, down projection: gate/up outputs f16 [pair][2][in_width]; the block
+                                       // computes hidden = swiglu(gate, up) of its pair itself.  Null: activations come from in / in_packed
+    const uint16_t* sigmoid;           // the sigmoid table swiglu uses (gu != null)
+    float swiglu_limit;
     uint16_t* out;                     // fp16
     int64_t out_pair_stride;           // halves between consecutive pairs
     int64_t out_slot_stride;           // halves between the outputs of consecutive slots of one pair

@@ -182,9 +182,9 @@ __global__ void __launch_bounds__(256) gemv_fast_kernel(mfq_amd_projection p, in
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
         const int token = first + n < batch ? first + n : batch - 1;
-        xs[n] = XSource{static_cast<const char*>(x) + static_cast<int64_t>(token) * x_stride * element, x_dtype, vector_ok != 0};
+        xs[n] = XSource{static_cast<const char*>(x) + static_cast<int64_t>(token) * x_stride * element, x_dtype, vector_ok != 0, nullptr};
     }
-    fast_rows<CLS, LPR, SLABS, NT, kRing, false, SLOTS>(ctx, xs, p.input_width, row_begin, row_end, p.output_rows,
+    fast_rows<CLS, LPR, SLABS, NT, kRing, kXRaw, SLOTS>(ctx, xs, p.input_width, row_begin, row_end, p.output_rows,
         [&](int n, int row, float value) { if (first + n < batch) y[static_cast<int64_t>(first + n) * y_stride + row] = value; });
 }
 

@@ -89,38 +89,94 @@ __global__ void __launch_bounds__(256) moe_rows_exact_kernel(RowsArgs a) {
 // One block = one routed pair x rows_per_block output rows of its expert; a quarter of the rows per
 // wave.  Pairs of one expert sit next to each other in the grid, and the same row tile of
 // neighbouring pairs lands on the same XCD, so an expert's weights come from HBM once.
-template <int CLS, int LPR, bool PACKED, int SLOTS, int IB>
+// LDS a block of the down projection keeps for the hidden row of its pair: the fp16 values, the largest magnitude
+// (as fp16 bits) and the normaliser {2^-e, 2^e} derived from it.
+struct HiddenLds {
+    uint16_t values[16 * kLaneColumns];
+    uint32_t wave_largest[4];
+    float scale[2];
+};
+
+// Every lane returns the largest value of the wave.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    auto step = [](uint32_t x, uint32_t other) { return other > x ? other : x; };
+    v = step(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, false)));
+    v = step(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, false)));
+    v = step(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x141, 0xF, 0xF, false)));
+    v = step(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x140, 0xF, 0xF, false)));
+    v = step(v, static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 16, kWave)));
+    v = step(v, static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 32, kWave)));
+    return v;
+}
+
+// hidden = swiglu(gate, up) of one routed pair, computed by the block that multiplies it: two columns per thread, the
+// row's largest magnitude per wave.  Contains one barrier; every thread of the block calls it once.
+__device__ __forceinline__ void hidden_to_lds(const RowsArgs& a, int pair, HiddenLds* hidden) {
+    const uint16_t* gate = a.gu + static_cast<int64_t>(pair) * 2 * a.in_width;
+    const uint16_t* up = gate + a.in_width;
+    uint32_t largest = 0u;
+    for (int col = threadIdx.x; col < a.in_width; col += blockDim.x) {
+        const uint16_t h = swiglu_bits(gate[col], up[col], a.swiglu_limit, a.sigmoid);
+        hidden->values[col] = h;
+        const uint32_t magnitude = h & 0x7fffu;
+        largest = magnitude > largest && magnitude <= 0x7c00u ? magnitude : largest;     // NaN does not count, as with fmaxf
+    }
+    largest = wave_max_u32(largest);       // the bits of non-negative halves order like their values
+    if (threadIdx.x % kWave == 0) hidden->wave_largest[threadIdx.x / kWave] = largest;
+    __syncthreads();
+}
+
+// One block = one routed pair x rows_per_block output rows of its expert; a quarter of the rows per
+// wave.  Pairs of one expert sit next to each other in the grid, and the same row tile of
+// neighbouring pairs lands on the same XCD, so an expert's weights come from HBM once.
+template <int CLS, int LPR, int XMODE, int SLOTS, int IB>
 __device__ __forceinline__ void rows_fast_pair(const RowsArgs& a, const mfq_amd_projection& pool, const PairItem& item, int slot,
-                                               unsigned char* lds) {
+                                               unsigned char* lds, HiddenLds* hidden) {
     const FastCtx<CLS> ctx = fast_ctx<CLS>(pool, item.local, lds);
     const int wave = uniform(static_cast<int>(threadIdx.x / kWave));
     const int rows_per_wave = a.rows_per_block / 4;
     const int row_begin = blockIdx.x * a.rows_per_block + wave * rows_per_wave;
-    if (row_begin >= a.out_rows) return;
-    const int row_end = row_begin + rows_per_wave < a.out_rows ? row_begin + rows_per_wave : a.out_rows;
     const int pair = item.pair;
+    // the hidden row of the pair: computed while the first packed rows are on their way
+    auto prologue = [&] {
+        if constexpr (XMODE == kXScaled) {
+            hidden_to_lds(a, pair, hidden);
+            if (threadIdx.x == 0) {
+                float down, up;
+                uint32_t largest = hidden->wave_largest[0];
+                for (int w = 1; w < 4; ++w) largest = hidden->wave_largest[w] > largest ? hidden->wave_largest[w] : largest;
+                normaliser(half_bits_to_float(static_cast<uint16_t>(largest)), down, up);
+                hidden->scale[0] = down; hidden->scale[1] = up;
+            }
+            __syncthreads();
+        }
+    };
+    if (row_begin >= a.out_rows) { prologue(); return; }
+    const int row_end = row_begin + rows_per_wave < a.out_rows ? row_begin + rows_per_wave : a.out_rows;
     uint16_t* out = a.out + (slot - a.slot_base) * a.out_slot_stride + pair * a.out_pair_stride;
     const int64_t source = a.in_per_pair ? pair : pair / a.top_k;
-    const XSource xs[1] = {{PACKED ? static_cast<const void*>(a.in_packed + source * a.in_packed_stride)
-                                   : pair_source(a, pair), a.in_dtype, a.in_vector_ok != 0}};
+    const XSource xs[1] = {{XMODE == kXPacked ? static_cast<const void*>(a.in_packed + source * a.in_packed_stride)
+                            : XMODE == kXScaled ? static_cast<const void*>(hidden->values) : pair_source(a, pair),
+                            XMODE == kXScaled ? MFQ_AMD_F16 : a.in_dtype, XMODE == kXScaled ? true : a.in_vector_ok != 0,
+                            hidden->scale}};
     constexpr int kRing = FastClass<CLS>::kRing < SLOTS || SLOTS == 0 ? FastClass<CLS>::kRing : SLOTS;
-    fast_rows<CLS, LPR, 1, 1, kRing, PACKED, SLOTS, IB>(ctx, xs, a.in_width, row_begin, row_end, a.out_rows,
-        [&](int, int row, float value) { out[row] = float_to_half_bits(value); });
+    fast_rows<CLS, LPR, 1, 1, kRing, XMODE, SLOTS, IB>(ctx, xs, a.in_width, row_begin, row_end, a.out_rows,
+        [&](int, int row, float value) { out[row] = float_to_half_bits(value); }, prologue);
 }
 
-template <int CLS, int LPR, bool PACKED, int SLOTS>
-__device__ __forceinline__ void rows_fast_block(const RowsArgs& a, const PairItem& item, int slot, unsigned char* lds) {
+template <int CLS, int LPR, int XMODE, int SLOTS>
+__device__ __forceinline__ void rows_fast_block(const RowsArgs& a, const PairItem& item, int slot, unsigned char* lds, HiddenLds* hidden) {
     const mfq_amd_projection& pool = a.pools[item.pool];
     if constexpr (FastClass<CLS>::kNvq) {
         nvq_fast_tables(pool, lds);
         __syncthreads();
         // the index width of the format fixes the bit positions of every index: one copy of the row loop each
         const int index_bits = nvq_format_index_bits(pool.format);
-        if (index_bits == 10) rows_fast_pair<CLS, LPR, PACKED, SLOTS, 10>(a, pool, item, slot, lds);
-        else if (index_bits == 9) rows_fast_pair<CLS, LPR, PACKED, SLOTS, 9>(a, pool, item, slot, lds);
-        else rows_fast_pair<CLS, LPR, PACKED, SLOTS, 8>(a, pool, item, slot, lds);
+        if (index_bits == 10) rows_fast_pair<CLS, LPR, XMODE, SLOTS, 10>(a, pool, item, slot, lds, hidden);
+        else if (index_bits == 9) rows_fast_pair<CLS, LPR, XMODE, SLOTS, 9>(a, pool, item, slot, lds, hidden);
+        else rows_fast_pair<CLS, LPR, XMODE, SLOTS, 8>(a, pool, item, slot, lds, hidden);
     } else {
-        rows_fast_pair<CLS, LPR, PACKED, SLOTS, 0>(a, pool, item, slot, lds);
+        rows_fast_pair<CLS, LPR, XMODE, SLOTS, 0>(a, pool, item, slot, lds, hidden);
     }
 }
 
@@ -128,21 +184,24 @@ __device__ __forceinline__ void rows_fast_block(const RowsArgs& a, const PairIte
 // (uniformly) into the kernel class of its expert's pool.
 // SLOTS: row slots per wave (a slot is one row for LPR 64 and four rows for LPR 16), so a block
 // covers 4 * SLOTS * (64 / LPR) rows; 0 = taken from rows_per_block at run time.
-template <int LPR, bool PACKED, int SLOTS>
+// XMODE: kXRaw / kXPacked: activations from RowsArgs::in / in_packed; kXScaled: the block computes the hidden row of
+// its pair from RowsArgs::gu first (down projection of the FFN; rows of at most 512 columns).
+template <int LPR, int XMODE, int SLOTS>
 __global__ void __launch_bounds__(256) moe_rows_fast_kernel(RowsArgs a) {
     // The NVQ tables sit in statically sized LDS: their addresses are then constants of the instruction
     // stream.  Four blocks of a CU hold 4 x 35 KB of the 160 KB, which the register budget allows anyway.
     __shared__ __attribute__((aligned(16))) unsigned char lds[kNvqFastLdsBytes];
+    __shared__ __attribute__((aligned(16))) HiddenLds hidden[1];
     const int slot = a.slot_base + blockIdx.z;
     const PairItem item = a.pair_items[static_cast<int64_t>(slot) * a.pairs + blockIdx.y];
     switch (item.cls) {
-        case K_NINT_2_16: rows_fast_block<K_NINT_2_16, LPR, PACKED, SLOTS>(a, item, slot, lds); break;
-        case K_NINT_3_24: rows_fast_block<K_NINT_3_24, LPR, PACKED, SLOTS>(a, item, slot, lds); break;
-        case K_NINT_4_24: rows_fast_block<K_NINT_4_24, LPR, PACKED, SLOTS>(a, item, slot, lds); break;
-        case K_NINT_4_32: rows_fast_block<K_NINT_4_32, LPR, PACKED, SLOTS>(a, item, slot, lds); break;
-        case K_NINT_8_48: rows_fast_block<K_NINT_8_48, LPR, PACKED, SLOTS>(a, item, slot, lds); break;
-        case K_NVQ_D4: rows_fast_block<K_NVQ_D4, LPR, PACKED, SLOTS>(a, item, slot, lds); break;
-        case K_MXFP4: rows_fast_block<K_MXFP4, LPR, PACKED, SLOTS>(a, item, slot, lds); break;
+        case K_NINT_2_16: rows_fast_block<K_NINT_2_16, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
+        case K_NINT_3_24: rows_fast_block<K_NINT_3_24, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
+        case K_NINT_4_24: rows_fast_block<K_NINT_4_24, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
+        case K_NINT_4_32: rows_fast_block<K_NINT_4_32, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
+        case K_NINT_8_48: rows_fast_block<K_NINT_8_48, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
+        case K_NVQ_D4: rows_fast_block<K_NVQ_D4, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
+        case K_MXFP4: rows_fast_block<K_MXFP4, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
         default: break;   // unrouted, exact-only pools and classes without a fast path
     }
 }
@@ -282,6 +341,8 @@ __global__ void shared_gate_kernel(const uint16_t* routed, const uint16_t* pairs
 }  // namespace dev
 
 namespace {
+constexpr int kFusedSwigluPairs = 100;   // up to this many routed pairs the down blocks compute their hidden rows themselves
+
 void launch_weighted_reduce(const uint16_t* pairs, const float* weights, const int32_t* ids, int experts, int tokens, int top_k,
                             int width, void* out, int out_dtype, hipStream_t stream) {
     // small outputs want many threads rather than wide ones
@@ -338,21 +399,26 @@ void launch_rows_fast(const RowsArgs& args, int slots, bool nvq, hipStream_t str
     const bool narrow = args.in_width <= 16 * dev::kLaneColumns;
     const int wave_slots = args.rows_per_block / (narrow ? 16 : 4);
     auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), bytes, stream, args); };
-    if (args.in_packed != nullptr) {
+    if (args.gu != nullptr) {
+        MFQ_REQUIRE(narrow && args.in_per_pair && args.sigmoid != nullptr, "the fused SwiGLU serves rows of at most 512 columns");
+        if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 4>);
+        else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 8>);
+        else launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 0>);
+    } else if (args.in_packed != nullptr) {
         // straight-line variants for the block heights the FFN uses, the looped kernel for the rest
         if (narrow) {
-            if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<16, true, 4>);
-            else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<16, true, 8>);
-            else launch(dev::moe_rows_fast_kernel<16, true, 0>);
+            if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 4>);
+            else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 8>);
+            else launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 0>);
         } else {
-            if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<64, true, 4>);
-            else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<64, true, 8>);
-            else if (wave_slots == 16) launch(dev::moe_rows_fast_kernel<64, true, 16>);
-            else launch(dev::moe_rows_fast_kernel<64, true, 0>);
+            if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<64, dev::kXPacked, 4>);
+            else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<64, dev::kXPacked, 8>);
+            else if (wave_slots == 16) launch(dev::moe_rows_fast_kernel<64, dev::kXPacked, 16>);
+            else launch(dev::moe_rows_fast_kernel<64, dev::kXPacked, 0>);
         }
     } else {
-        if (narrow) launch(dev::moe_rows_fast_kernel<16, false, 0>);
-        else launch(dev::moe_rows_fast_kernel<64, false, 0>);
+        if (narrow) launch(dev::moe_rows_fast_kernel<16, dev::kXRaw, 0>);
+        else launch(dev::moe_rows_fast_kernel<64, dev::kXRaw, 0>);
     }
     check_launch("moe_rows_fast_kernel");
 }
@@ -708,7 +774,12 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         x.direct_pairs = !x.pairs_only && decode && tokens <= 4 && !x.want_items && f->d_expert_info != nullptr && f->config.launch_mode == 0;
         const bool fast_mode = decode && f->config.launch_mode == 0;
         const bool pack_x = fast_mode && f->d_x_packed != nullptr;
-        const bool pack_hidden = fast_mode && f->d_hidden_packed != nullptr;
+        // the down blocks compute the hidden row of their pair themselves when nothing else reads it
+        // (every block of a pair repeats the SwiGLU and the packing of its row: worth a kernel less up to about a hundred
+        // pairs; measured at 512 experts x (2048 <-> 512), top-10: batch 1 -4 us, batch 4 -5 us per step, batch 16 +0.5 us)
+        const bool fuse_swiglu = fast_mode && !f->decode_needs_items && I <= 16 * dev::kLaneColumns && rows_fast_geometry(I, MFQ_AMD_F16) &&
+                                 pairs <= kFusedSwigluPairs;
+        const bool pack_hidden = fast_mode && !fuse_swiglu && f->d_hidden_packed != nullptr;
         if (pack_x) {
             plan.pack.src = x_dev; plan.pack.dst = f->d_x_packed; plan.pack.stride = dev::xpack_row_dwords(H);
             plan.pack.rows = tokens; plan.pack.width = H; plan.pack.dtype = f->config.x_dtype;
@@ -797,7 +868,9 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
 
         const bool hidden_tiles = !decode && f->config.launch_mode == 0 && f->d_expert_info != nullptr &&
                                   tiles_fast_geometry(I, MFQ_AMD_F16, 1);
-        if (hidden_tiles) {
+        if (fuse_swiglu) {
+            // no kernel of its own
+        } else if (hidden_tiles) {
             launch_swiglu_tiles(f->d_gu, f->d_gu + I, 2 * static_cast<int64_t>(I), I, pairs, f->config.swiglu_limit, f->d_sigmoid,
                                 ids_dev, f->d_expert_info + 2 * static_cast<int64_t>(E), E, f->d_hidden, stream);
         } else if (pack_hidden) {
@@ -821,6 +894,7 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         rows.out = f->d_pairs; rows.out_pair_stride = H; rows.out_slot_stride = 0;
         rows.slot_base = 2; rows.out_rows = H;
         rows.in_packed = pack_hidden ? f->d_hidden_packed : nullptr; rows.in_packed_stride = dev::xpack_row_dwords(I);
+        if (fuse_swiglu) { rows.gu = f->d_gu; rows.sigmoid = f->d_sigmoid; rows.swiglu_limit = f->config.swiglu_limit; }
         rows.in_tiles = hidden_tiles ? f->d_hidden : nullptr; rows.in_tiles_layout_stride = 0;
         run_rows(2, 3);
         f->mark(4, stream);
