@@ -217,6 +217,11 @@ int mfq_amd_moe_ffn_run(mfq_amd_moe_ffn* ffn, const void* x_dev, const int32_t* 
 int mfq_amd_moe_ffn_run_logits(mfq_amd_moe_ffn* ffn, const void* x_dev, const void* logits_dev, int32_t logits_dtype,
                                int32_t normalize, float norm_floor, float scale, int32_t tokens, void* out_dev,
                                void* stream);
+/* The same with the router matmul in front: logits = x . router^T (as mfq_amd_router_logits, into a buffer of the
+ * object), then mfq_amd_moe_ffn_run_logits.  router_dev[experts, hidden].  Replaces the router GEMM + moe_topk_cuda +
+ * MfeFfnRuntime::run sequence of FFN::forward_impl (cpp_runtime/backends/cuda/core/ffn.cpp:443-447, :676-835). */
+int mfq_amd_moe_ffn_run_router(mfq_amd_moe_ffn* ffn, const void* x_dev, const void* router_dev, int32_t router_dtype,
+                               int32_t normalize, float norm_floor, float scale, int32_t tokens, void* out_dev, void* stream);
 /* Routes of the last mfq_amd_moe_ffn_run_logits: ids i32 [tokens, k], weights f32 [tokens, k]. */
 int mfq_amd_moe_ffn_routes(mfq_amd_moe_ffn* ffn, const int32_t** ids_dev, const float** weights_dev);
 /* Stage buffers of the last run (device pointers, valid until destroy): gate_up f16 [tokens, k, 2, I]

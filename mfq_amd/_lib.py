@@ -78,6 +78,8 @@ EXPORTS = {
     "mfq_amd_moe_ffn_create": (C.c_int, [C.POINTER(MoeFfnConfig), c_void_pp]),
     "mfq_amd_moe_ffn_run_logits": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_float, C.c_float,
                                             C.c_int32, C.c_void_p, C.c_void_p]),
+    "mfq_amd_moe_ffn_run_router": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_float, C.c_float,
+                                            C.c_int32, C.c_void_p, C.c_void_p]),
     "mfq_amd_moe_ffn_routes": (C.c_int, [C.c_void_p, c_void_pp, c_void_pp]),
     "mfq_amd_moe_ffn_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p,
                                       C.c_void_p]),

@@ -593,6 +593,7 @@ struct mfq_amd_moe_ffn {
     uint16_t *d_gu = nullptr, *d_hidden = nullptr, *d_pairs = nullptr;
     const uint16_t* d_sigmoid = nullptr;   // the device's table: not owned
     int32_t* d_wave_base = nullptr;      // scratch of the two-kernel route plan
+    float* d_logits = nullptr;           // router logits of run_router
     int32_t* d_route_ids = nullptr;      // routes selected by run_logits
     float* d_route_weights = nullptr;
     uint32_t *d_x_packed = nullptr, *d_hidden_packed = nullptr;
@@ -609,7 +610,7 @@ struct mfq_amd_moe_ffn {
     ~mfq_amd_moe_ffn() {
         void* all[] = {d_pools, d_pool_class, d_pool_bytes, d_expert_pool, d_expert_info, d_expert_words, d_item_info, d_pair_items, d_items, d_class_offsets, d_tile_items,
                        d_tile_offsets, d_counts, d_bounds, d_tile_bounds, d_tile_experts, d_ids_dst, d_distinct,
-                       d_touched, d_gu, d_hidden, d_pairs, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base};
+                       d_touched, d_gu, d_hidden, d_pairs, d_logits, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base};
         for (void* p : all) if (p) (void)hipFree(p);
         for (hipEvent_t e : events) if (e) (void)hipEventDestroy(e);
     }
@@ -708,6 +709,7 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
         f->d_hidden = device_alloc<uint16_t>(pairs * f->intermediate);
         f->d_pairs = device_alloc<uint16_t>(pairs * f->hidden);
         f->d_sigmoid = device_state().sigmoid_table;
+        f->d_logits = device_alloc<float>(static_cast<size_t>(c.max_tokens) * E);
         f->d_route_ids = device_alloc<int32_t>(pairs);
         f->d_route_weights = device_alloc<float>(pairs);
         f->d_wave_base = device_alloc<int32_t>(static_cast<size_t>(kPlanThreads / 64) * E);
@@ -937,6 +939,21 @@ extern "C" int mfq_amd_moe_ffn_run_logits(mfq_amd_moe_ffn* f, const void* x_dev,
         }
         ffn_run(f, x_dev, f->d_route_ids, f->d_route_weights, tokens, out_dev, stream, fused ? &route : nullptr);
     });
+}
+
+extern "C" int mfq_amd_moe_ffn_run_router(mfq_amd_moe_ffn* f, const void* x_dev, const void* router_dev, int32_t router_dtype,
+                                          int32_t normalize, float norm_floor, float scale, int32_t tokens, void* out_dev,
+                                          void* stream_ptr) {
+    const int status = guarded([&] {
+        MFQ_REQUIRE(f && x_dev && router_dev && out_dev, "null argument");
+        MFQ_REQUIRE(tokens >= 0 && tokens <= f->max_tokens, "token count exceeds the workspace capacity");
+        MFQ_REQUIRE(router_dtype >= MFQ_AMD_F32 && router_dtype <= MFQ_AMD_BF16, "router weights must be float32, float16 or bfloat16");
+        if (tokens == 0) return;
+        launch_router_logits(x_dev, f->config.x_dtype, router_dev, router_dtype, tokens, f->experts, f->hidden, f->d_logits,
+                             as_stream(stream_ptr));
+    });
+    if (status != MFQ_AMD_OK || tokens == 0) return status;
+    return mfq_amd_moe_ffn_run_logits(f, x_dev, f->d_logits, MFQ_AMD_F32, normalize, norm_floor, scale, tokens, out_dev, stream_ptr);
 }
 
 extern "C" int mfq_amd_moe_ffn_routes(mfq_amd_moe_ffn* f, const int32_t** ids_dev, const float** weights_dev) {

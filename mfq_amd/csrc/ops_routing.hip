@@ -50,6 +50,82 @@ __global__ void __launch_bounds__(64) router_logits_kernel(const void* x, int x_
     if (e0 + lane < experts) logits[static_cast<int64_t>(token) * experts + e0 + lane] = sum;
 }
 
+// The same logits for fp16 / bf16 operands, one thread per (token, expert).  The product of two such values is exact
+// in fp32, so a fused multiply-add gives the very sum of the separate multiply and add above (products below 2^-126
+// excepted, which cannot move a sum of ordinary magnitude); what remains is the chain of `width` dependent additions
+// the fixed order asks for, and every chain has a thread of its own.  A block = 64 experts x 4 tokens (one wave per
+// token): the router rows pass through LDS in tiles of 128 columns, loaded with coalesced 16-byte requests one tile
+// ahead of their use; a wave's activations are wave-uniform.
+constexpr int kRouterTile = 64;                        // columns per LDS tile
+constexpr int kRouterPitch = kRouterTile * 4 + 16;     // bytes per expert row in LDS (fp32): the pad keeps 16-byte reads conflict-free
+__global__ void __launch_bounds__(256) router_logits_chain_kernel(const uint16_t* x, int x_half, const uint16_t* router, int router_half,
+                                                                  int tokens, int experts, int width, float* logits) {
+    // Both operands are widened to fp32 once, by the thread that stages them: a single wave per SIMD issues an
+    // instruction every five cycles or so, so the inner loop is kept to the fused multiply-add and its LDS reads.
+    __shared__ __attribute__((aligned(16))) unsigned char tile[2][64 * kRouterPitch];
+    __shared__ __attribute__((aligned(16))) float x_tile[2][4 * kRouterTile];      // the four tokens' columns of the tile
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int e0 = blockIdx.x * 64;
+    const int token = blockIdx.y * 4 + wave;
+    auto widen = [](uint32_t bits, int half) { return half ? half_bits_to_float(static_cast<uint16_t>(bits)) : bits_to_float(bits << 16); };
+    // staging role: thread -> rows tid / 8 and tid / 8 + 32 of the tile, its 16-byte piece tid % 8 (eight columns)
+    const int piece = tid & 7, first_row = tid >> 3;
+    uint4 staged[2], staged_x = {0u, 0u, 0u, 0u};
+    const int x_token = blockIdx.y * 4 + (tid >> 3) < tokens ? blockIdx.y * 4 + (tid >> 3) : tokens - 1;   // threads 0..31: token tid / 8
+    auto load_tile = [&](int c0) {
+        if (tid < 32) staged_x = *reinterpret_cast<const uint4*>(x + static_cast<int64_t>(x_token) * width + c0 + piece * 8);
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int row = first_row + 32 * k;
+            const int expert = e0 + row < experts ? e0 + row : experts - 1;
+            staged[k] = *reinterpret_cast<const uint4*>(router + static_cast<int64_t>(expert) * width + c0 + piece * 8);
+        }
+    };
+    auto store_wide = [&](const uint4& v, int half, float* to) {
+        const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+        float4 lo, hi;
+        lo.x = widen(words[0] & 0xffffu, half); lo.y = widen(words[0] >> 16, half);
+        lo.z = widen(words[1] & 0xffffu, half); lo.w = widen(words[1] >> 16, half);
+        hi.x = widen(words[2] & 0xffffu, half); hi.y = widen(words[2] >> 16, half);
+        hi.z = widen(words[3] & 0xffffu, half); hi.w = widen(words[3] >> 16, half);
+        reinterpret_cast<float4*>(to)[0] = lo;
+        reinterpret_cast<float4*>(to)[1] = hi;
+    };
+    auto store_tile = [&](int buffer) {
+        if (tid < 32) store_wide(staged_x, x_half, &x_tile[buffer][(tid >> 3) * kRouterTile + piece * 8]);
+#pragma unroll
+        for (int k = 0; k < 2; ++k)
+            store_wide(staged[k], router_half, reinterpret_cast<float*>(tile[buffer] + (first_row + 32 * k) * kRouterPitch) + piece * 8);
+    };
+    const int full = width / kRouterTile * kRouterTile;          // columns covered by whole tiles
+    float sum = 0.0f;
+    if (full > 0) load_tile(0);
+    for (int c0 = 0; c0 < full; c0 += kRouterTile) {
+        const int buffer = (c0 / kRouterTile) & 1;
+        store_tile(buffer);
+        __syncthreads();
+        if (c0 + kRouterTile < full) load_tile(c0 + kRouterTile);
+        const float* mine = reinterpret_cast<const float*>(tile[buffer] + lane * kRouterPitch);
+        const float* xs = &x_tile[buffer][wave * kRouterTile];
+#pragma unroll
+        for (int c = 0; c < kRouterTile; c += 4) {
+            const float4 wv = *reinterpret_cast<const float4*>(mine + c);
+            const float4 xv = *reinterpret_cast<const float4*>(xs + c);
+            sum = fmaf(xv.x, wv.x, sum);
+            sum = fmaf(xv.y, wv.y, sum);
+            sum = fmaf(xv.z, wv.z, sum);
+            sum = fmaf(xv.w, wv.w, sum);
+        }
+        // the buffer written two tiles from now is the one just read: every wave must be done with it first
+        __syncthreads();
+    }
+    const int expert = e0 + lane;
+    const uint16_t* w = router + static_cast<int64_t>(expert < experts ? expert : experts - 1) * width;
+    const uint16_t* xr = x + static_cast<int64_t>(token < tokens ? token : tokens - 1) * width;
+    for (int c = full; c < width; ++c) sum = fmaf(widen(xr[c], x_half), widen(w[c], router_half), sum);
+    if (expert < experts && token < tokens) logits[static_cast<int64_t>(token) * experts + expert] = sum;
+}
+
 // ------------------------------------------------------------- top-k ----
 __device__ __forceinline__ float load_logit(const void* logits, int dtype, int64_t index) {
     float raw;
@@ -950,6 +1026,24 @@ __global__ void __launch_bounds__(kPlanThreads) touched_bytes_kernel(const int32
 
 }  // namespace dev
 
+void launch_router_logits(const void* x, int x_dtype, const void* router, int router_dtype, int tokens, int experts, int width,
+                          float* logits, hipStream_t stream) {
+    if (x_dtype != MFQ_AMD_F32 && router_dtype != MFQ_AMD_F32) {
+        // products of 16-bit operands are exact: one chain per thread
+        const bool aligned = width % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(router) % 16 == 0;
+        if (aligned) {
+            hipLaunchKernelGGL(dev::router_logits_chain_kernel, dim3((experts + 63) / 64, (tokens + 3) / 4), dim3(256), 0, stream,
+                               static_cast<const uint16_t*>(x), x_dtype == MFQ_AMD_F16 ? 1 : 0, static_cast<const uint16_t*>(router),
+                               router_dtype == MFQ_AMD_F16 ? 1 : 0, tokens, experts, width, logits);
+            check_launch("router_logits_chain_kernel");
+            return;
+        }
+    }
+    hipLaunchKernelGGL(dev::router_logits_kernel, dim3((experts + 63) / 64, tokens), dim3(64), 0, stream, x, x_dtype, router,
+                       router_dtype, experts, width, logits);
+    check_launch("router_logits_kernel");
+}
+
 void launch_touched_bytes(const int32_t* ids, int pairs, int experts, int slots, const ExpertInfo* expert_info,
                           int64_t* touched_bytes, int32_t* distinct, hipStream_t stream) {
     MFQ_REQUIRE(experts > 0 && experts <= kPlanMaxExperts && pairs >= 0, "invalid routing geometry");
@@ -1039,9 +1133,7 @@ extern "C" int mfq_amd_router_logits(const void* x_dev, int32_t x_dtype, const v
         MFQ_REQUIRE(tokens >= 0 && experts > 0 && width > 0, "invalid router geometry");
         MFQ_REQUIRE(x_dtype >= 0 && x_dtype <= 2 && router_dtype >= 0 && router_dtype <= 2, "unknown dtype");
         if (!tokens) return;
-        hipLaunchKernelGGL(dev::router_logits_kernel, dim3((experts + 63) / 64, tokens), dim3(64), 0, as_stream(stream),
-                           x_dev, x_dtype, router_dev, router_dtype, experts, width, logits_dev);
-        check_launch("router_logits_kernel");
+        launch_router_logits(x_dev, x_dtype, router_dev, router_dtype, tokens, experts, width, logits_dev, as_stream(stream));
     });
 }
 

@@ -123,6 +123,9 @@ struct PlanArgs {
 };
 
 void launch_route_plan(const PlanArgs& args, hipStream_t stream);
+// logits[tokens, experts] = x . router^T in fp32, columns added in ascending order per output.
+void launch_router_logits(const void* x, int x_dtype, const void* router, int router_dtype, int tokens, int experts, int width,
+                          float* logits, hipStream_t stream);
 // touched_bytes[0] = packed bytes of the distinct experts `ids` names over the slots of expert_info; distinct[0] = their number.
 void launch_touched_bytes(const int32_t* ids, int pairs, int experts, int slots, const ExpertInfo* expert_info,
                           int64_t* touched_bytes, int32_t* distinct, hipStream_t stream);

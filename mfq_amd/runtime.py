@@ -260,6 +260,19 @@ class MfeFfnRuntime:
                                                    int(normalize), norm_floor, scale, tokens, out.data_ptr(), _stream()))
         return out
 
+    def run_router(self, x: torch.Tensor, router: torch.Tensor, out: torch.Tensor | None = None, normalize: bool = True,
+                   norm_floor: float = 1e-20, scale: float = 1.0) -> torch.Tensor:
+        """Router matmul, top-k routing and the layer in one call."""
+        if x.dtype != self.x_dtype:
+            raise ValueError(f"x must be {self.x_dtype}")
+        x, router = x.contiguous(), router.contiguous()
+        tokens = x.shape[0]
+        if out is None:
+            out = torch.empty((tokens, self.hidden), dtype=self.out_dtype, device="cuda")
+        L.check(L.lib().mfq_amd_moe_ffn_run_router(self._handle, x.data_ptr(), router.data_ptr(), _dtype_code(router),
+                                                   int(normalize), norm_floor, scale, tokens, out.data_ptr(), _stream()))
+        return out
+
     def routes(self, tokens: int) -> tuple[torch.Tensor, torch.Tensor]:
         """Copies of the ids and weights the last run_logits selected."""
         ids, weights = C.c_void_p(), C.c_void_p()

@@ -199,6 +199,29 @@ def test_layer_with_fused_routing_equals_topk_then_layer(tokens, experts, k):
     assert rel_l2(got, expect) <= FFN_TOL
 
 
+@pytest.mark.parametrize("tokens", [1, 9, 48])
+def test_layer_with_the_router_matmul_in_front(tokens):
+    """run_router = router matmul + top-k + layer in one call: same routes and output as the three calls."""
+    import torch
+    from mfq_amd import runtime as R, synth
+    experts, hidden, inter, k = 24, 512, 128, 6
+    tensors, runtimes, _ = _layer("test/moe/random", experts, hidden, inter, "random")
+    x = synth.to_bf16(synth.normal(f"test/moe/router/x/{tokens}", (tokens, hidden)))
+    router = synth.to_bf16(synth.normal("test/moe/router/w", (experts, hidden), 0.02))
+    xd = torch.from_numpy(x).to(torch.bfloat16).cuda()
+    rd = torch.from_numpy(router).to(torch.bfloat16).cuda()
+    ffn = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=64)
+    ids, weights = R.moe_topk(R.router_logits(xd, rd), k)
+    want = ffn.run(xd, ids, weights).cpu().numpy()
+    got = ffn.run_router(xd, rd).cpu().numpy()
+    got_ids, got_weights = ffn.routes(tokens)
+    ids_ref, weights_ref = O.topk(O.router_logits(x, router), k)
+    np.testing.assert_array_equal(got_ids.numpy(), ids_ref)
+    np.testing.assert_array_equal(got_ids.numpy(), ids.cpu().numpy())
+    np.testing.assert_array_equal(got, want)
+    assert rel_l2(got, oracle_layer(x, ids_ref, weights_ref, tensors)) <= FFN_TOL
+
+
 def test_decode_layer_replayed_from_a_hip_graph():
     """The layer allocates nothing and synchronises nothing: captured once, every replay (with eager work and
     synchronisation in between) gives the eager result, for the id-based and the logits-based entry."""

@@ -150,3 +150,19 @@ def test_topk_many_random_rows(seed):
     logits = rng.normal(0, [0.02, 1.0, 8.0][seed], (257, 512)).astype(np.float32)
     _check_topk(logits, 10)
     _check_topk(logits[:33, :256].copy(), 8)
+
+
+@pytest.mark.parametrize("x_dtype,r_dtype", [("f16", "f16"), ("bf16", "f16"), ("f32", "bf16"), ("f32", "f32")])
+def test_router_logits_every_operand_type(x_dtype, r_dtype):
+    """16-bit operands take the kernel with one thread per logit (fused multiply-add of an exact product), float32
+    operands the kernel with separate multiply and add; both give the oracle's sums bit for bit."""
+    import torch
+    from mfq_amd import runtime as R
+    rng = np.random.default_rng(77)
+    types = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
+    for tokens, experts, width in ((3, 300, 512), (2, 64, 72), (1, 7, 33)):
+        x = torch.from_numpy(rng.normal(0, 1, (tokens, width)).astype(np.float32)).to(types[x_dtype])
+        router = torch.from_numpy(rng.normal(0, 0.05, (experts, width)).astype(np.float32)).to(types[r_dtype])
+        expect = O.router_logits(x.float().numpy(), router.float().numpy())
+        got = R.router_logits(x.cuda(), router.cuda()).cpu().numpy()
+        assert bits_equal(got, expect), (x_dtype, r_dtype, tokens, experts, width)
