@@ -24,6 +24,7 @@ from pathlib import Path
 
 ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "tests"))      # the synthetic workloads (synth.py, benchdata.py) live beside the tests
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
@@ -47,7 +48,8 @@ def parse_args():
 def make_inputs(tag, tokens, batches):
     """Per batch: bf16 activations, fp32 router logits (fixed-order dot on the GPU)."""
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     router = torch.from_numpy(synth.to_bf16(synth.normal(f"{tag}/router", (EXPERTS, HIDDEN), 0.02))).to(torch.bfloat16).cuda()
     xs, logits = [], []
     for b in range(batches):
@@ -57,13 +59,17 @@ def make_inputs(tag, tokens, batches):
     return xs, logits
 
 
-def decode_workload(batch, steps, warmup, launch_mode, layers=2, batches=8):
+def decode_workload(batch, steps, warmup, launch_mode, layers=2, batches=8, uniform=None):
+    """uniform: one format for every projection (config 3: "NINT4"); default: the drawn mix of config 4."""
     import torch
-    from mfq_amd import benchdata, runtime as R, synth
-    formats = [synth.draw_formats(f"cfg4/format/{p}", EXPERTS) for p in ("gate", "up", "down")]
-    copies = [benchdata.device_layer(f"cfg4/layer{i}", EXPERTS, HIDDEN, INTER, formats) for i in range(layers)]
+    from mfq_amd import runtime as R
+    import benchdata
+    import synth
+    tag = "cfg3" if uniform else "cfg4"
+    formats = [[uniform] * EXPERTS if uniform else synth.draw_formats(f"cfg4/format/{p}", EXPERTS) for p in ("gate", "up", "down")]
+    copies = [benchdata.device_layer(f"{tag}/layer{i}", EXPERTS, HIDDEN, INTER, formats) for i in range(layers)]
     ffns = [R.MfeFfnRuntime(*layer, top_k=TOP_K, max_tokens=max(batch, 16), launch_mode=launch_mode) for layer in copies]
-    xs, logits = make_inputs("cfg4", batch, batches)
+    xs, logits = make_inputs(tag, batch, batches)
     outs = [torch.empty((batch, HIDDEN), dtype=torch.float32, device="cuda") for _ in range(batches)]
     ids = [torch.empty((batch, TOP_K), dtype=torch.int32, device="cuda") for _ in range(batches)]
     weights = [torch.empty((batch, TOP_K), dtype=torch.float32, device="cuda") for _ in range(batches)]
@@ -152,58 +158,63 @@ def stage_bytes(work, step_index):
     return gu, dn, len(distinct)
 
 
-def cpu_baseline(work, budget_s=12.0):
-    """The same layer on the host cores: routed expert FFNs of batch 0 through the reference's own
-    AVX2 rows kernels on its pinned expert pool (NINT, NVQ) and the C restatement (MXFP4 rows,
-    SwiGLU chain).  Repeats until about `budget_s` seconds of CPU time have been spent."""
+def cpu_baseline(work, samples=7, budget_s=25.0):
+    """The same layer on the host cores, timed inside one C call per layer (oracle/ref_shim.cpp: ref_layer): the routed
+    expert FFNs of token batch 0 through the reference's own AVX2 rows kernels (NINT, NVQ) and the C restatement (MXFP4
+    rows, SwiGLU chain).  Median of `samples` calls on the reference's pinned expert pool (all cores) and on one
+    thread, as bench/cpu_nvq_bench.cpp:79-119 reports both; the one-thread samples stop early when the budget is spent."""
     import numpy as np
     from oracle import oracle as O
     gate, up, down = work["copies"][0]
     ids = work["ids"][0].cpu().numpy()
     x = work["xs"][0].float().cpu().numpy()
     tokens = ids.shape[0]
-    ref = O.ref_lib()
     by_expert = {}
     for t in range(tokens):
         for r in range(ids.shape[1]):
             by_expert.setdefault(int(ids[t, r]), []).append(t)
     layouts = {e: tuple(tn.host_layout(e) for tn in (gate, up, down)) for e in by_expert}
-    projections = {e: tuple(O.Projection(L) for L in layouts[e]) for e in by_expert}
+    ref = O.ref_lib()
+    sample = (f"the batch-{tokens} layer of token batch 0 ({len(by_expert)} distinct experts, {tokens * ids.shape[1]} routed pairs), "
+              f"one C call per layer")
+    if ref is None or not hasattr(ref, "ref_layer"):
+        # the C restatement alone, expert by expert (one thread)
+        projections = {e: tuple(O.Projection(L) for L in layouts[e]) for e in by_expert}
+        def once():
+            for e, toks in by_expert.items():
+                O.expert_ffn(*projections[e], x[toks], order=0)
+        once()
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter(); once(); times.append(time.perf_counter() - t0)
+        return {"value": tokens / float(np.median(times)), "unit": "tok/s", "cores": 1, "kind": "port", "samples": len(times),
+                "sample": sample + "; C restatement of the reference's CPU path"}
+    layer = O.RefLayer(layouts, by_expert, x)
 
-    def rows(e, which, inp):
-        L = layouts[e][which]
-        if ref is not None and L["family"] == 1:
-            return O.ref_nint_rows_pooled(L, inp)
-        if ref is not None and L["family"] == 2:
-            return O.ref_nvq_rows(L, inp, pooled=True)
-        return projections[e][which].rows(inp)
+    def timed(pooled, limit_s):
+        layer.run(pooled)                                   # warm: page in the weights, start the pool
+        times, spent = [], 0.0
+        while len(times) < samples and (len(times) < 3 or spent < limit_s):
+            t0 = time.perf_counter(); layer.run(pooled); dt = time.perf_counter() - t0
+            times.append(dt); spent += dt
+        return float(np.median(times)), len(times)
 
-    def layer_once():
-        for e, toks in by_expert.items():
-            inp = np.ascontiguousarray(x[toks])
-            g = rows(e, 0, inp).astype(np.float16)
-            u = rows(e, 1, inp).astype(np.float16)
-            hidden = O.swiglu_array(g, u)
-            rows(e, 2, hidden.astype(np.float32))
-
-    layer_once()
-    start, reps = time.perf_counter(), 0
-    while time.perf_counter() - start < budget_s:
-        layer_once()
-        reps += 1
-    elapsed = time.perf_counter() - start
-    kind = "reference" if ref is not None else "port"
-    cores = int(ref.ref_pool_participants()) if ref is not None else 1
-    return {"value": tokens * reps / elapsed, "unit": "tok/s", "cores": cores, "kind": kind,
-            "sample": f"{reps} repeats of the batch-{tokens} layer of batch 0 ({len(by_expert)} distinct experts, "
-                      f"{tokens * ids.shape[1]} routed pairs); NINT and NVQ rows through the reference library on its pinned pool, "
-                      f"MXFP4 rows and the SwiGLU chain through the C restatement"}
+    all_s, all_n = timed(True, budget_s * 0.4)
+    one_s, one_n = timed(False, budget_s * 0.6)
+    cores = int(ref.ref_pool_participants())
+    return {"value": tokens / all_s, "unit": "tok/s", "cores": cores, "kind": "reference", "samples": all_n,
+            "ms_per_layer": all_s * 1e3,
+            "one_thread": {"value": tokens / one_s, "unit": "tok/s", "cores": 1, "samples": one_n, "ms_per_layer": one_s * 1e3},
+            "sample": sample + "; NINT and NVQ rows through the reference library (all cores: its pinned expert pool), MXFP4 rows and "
+                               "the SwiGLU chain through the C restatement; median"}
 
 
-def prefill_measure(tokens=4096, reps=3):
+def prefill_measure(tokens=4096, reps=7):
     import numpy as np
     import torch
-    from mfq_amd import benchdata, runtime as R, synth
+    from mfq_amd import runtime as R
+    import benchdata
+    import synth
     formats = [synth.draw_formats(f"cfg4/format/{p}", EXPERTS) for p in ("gate", "up", "down")]
     layer = benchdata.device_layer("cfg5/layer", EXPERTS, HIDDEN, INTER, formats)
     ffn = R.MfeFfnRuntime(*layer, top_k=TOP_K, max_tokens=tokens)
@@ -214,55 +225,72 @@ def prefill_measure(tokens=4096, reps=3):
     ffn.run(x, ids, w, out)
     torch.cuda.synchronize()
     ffn.enable_timing(True)
-    best = None
+    runs = []
     for _ in range(reps):
         ffn.run(x, ids, w, out)
-        t = ffn.stage_times()
-        if best is None or sum(t.values()) < sum(best.values()):
-            best = t
+        runs.append(ffn.stage_times())
+    runs.sort(key=lambda t: t["gate_up"] + t["down"])
+    best = runs[len(runs) // 2]                       # the median run by grouped-GEMM time
     flops = tokens * TOP_K * 6.0 * HIDDEN * INTER
     gemm_ms = best["gate_up"] + best["down"]
     total_ms = sum(best.values())
     return {"tokens": tokens, "ms_layer": total_ms, "ms_gemm": gemm_ms, "tok_per_s": tokens / (total_ms / 1e3),
             "tflops_gemm": flops / (gemm_ms / 1e3) / 1e12, "mfma_frac_of_f16_peak": flops / (gemm_ms / 1e3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
-            "stages_ms": best, "element_type": "fp16 tiles, fp32 accumulate"}
+            "stages_ms": best, "element_type": "fp16 tiles, fp32 accumulate", "samples": reps, "statistic": "median run"}
 
 
-def gemv_measure():
-    """Configs 1 and 2: single dense GEMV 4096 x 4096, packed by this package's packers would take
-    minutes on the host, so random codes of the same layout are used."""
-    import torch
-    from mfq_amd import benchdata, runtime as R, synth
+def gemv_measure(calls=64):
+    """Configs 1 and 2: single dense GEMV 4096 x 4096 (random codes in the runtime layout: packing 16 M weights with
+    the Python packers takes minutes).  Every call reads another copy of the matrix; the copies add up to more than
+    the 256 MB last-level cache, and a HIP graph of `calls` calls is replayed between events, so the figure is an HBM
+    figure (bench/hip_nint_bench.cpp:58-86 times graph replays the same way)."""
     import ctypes as C
+    import torch
     from mfq_amd import _lib as L
+    import benchdata
+    import synth
     results = {}
     for name, fmt, batch in (("cfg1_nint4_32_b1", "NINT4-32", 1), ("cfg2_nvq3_b1", "NVQ3", 1), ("cfg2_nvq3_b8", "NVQ3", 8)):
-        pools = [benchdata.device_pool(fmt, [0], 1, 4096, 4096, synth.tensor_seed(f"{name}/{i}")) for i in range(12)]
+        first = benchdata.device_pool(fmt, [0], 1, 4096, 4096, synth.tensor_seed(f"{name}/0"))
+        copies = int(280e6 // first.nbytes()) + 1
+        pools = [first] + [benchdata.device_pool(fmt, [0], 1, 4096, 4096, synth.tensor_seed(f"{name}/{i}")) for i in range(1, copies)]
         x = torch.randn((batch, 4096), device="cuda").to(torch.bfloat16)
         y = torch.empty((batch, 4096), dtype=torch.float32, device="cuda")
-        stream = torch.cuda.current_stream().cuda_stream
+        stream = torch.cuda.Stream()
 
-        def run(i):
+        def run(i, handle):
             p = pools[i % len(pools)]
-            L.check(L.lib().mfq_amd_gemv(C.byref(p.view), 0, x.data_ptr(), L.BF16, batch, 4096, y.data_ptr(), 4096, stream))
+            L.check(L.lib().mfq_amd_gemv(C.byref(p.view), 0, x.data_ptr(), L.BF16, batch, 4096, y.data_ptr(), 4096, handle))
 
-        for i in range(12):
-            run(i)
-        torch.cuda.synchronize()
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        n = 48
-        for i in range(n):
-            run(i)
-        stop.record()
-        torch.cuda.synchronize()
-        us = start.elapsed_time(stop) / n * 1e3
-        v = pools[0].view
+        with torch.cuda.stream(stream):
+            for i in range(len(pools)):
+                run(i, stream.cuda_stream)
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(calls):
+                    run(i, torch.cuda.current_stream().cuda_stream)
+            graph.replay()
+            stream.synchronize()
+            times = []
+            for _ in range(7):
+                start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record(stream)
+                graph.replay()
+                stop.record(stream)
+                stream.synchronize()
+                times.append(start.elapsed_time(stop) / calls * 1e3)
+        us = sorted(times)[len(times) // 2]
+        v = first.view
         if v.family == 1:
             nbytes = 4096 * ((v.groups * v.group_size * 4 + 7) // 8 + 2 * v.groups + 17)
         else:
             nbytes = (4096 * (v.nvec * 8 + v.nsign * 7 + v.groups * 4) + 7) // 8 + 4096 * 4
-        results[name] = {"us": us, "weight_bytes": nbytes, "GBps": nbytes / us / 1e3, "frac_hbm": nbytes / us / 1e3 / HBM_PEAK_GBS}
+        results[name] = {"us": us, "weight_bytes": nbytes, "GBps": nbytes / us / 1e3, "frac_hbm": nbytes / us / 1e3 / HBM_PEAK_GBS,
+                         "rotation": f"{len(pools)} copies of the matrix ({len(pools) * first.nbytes() / 1e6:.0f} MB)",
+                         "timing": f"median of 7 replays of a HIP graph of {calls} calls"}
+        del pools
+        torch.cuda.empty_cache()
     return results
 
 
@@ -319,7 +347,8 @@ def main():
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic (random codes in the runtime packed layout, N(0,1) bf16 activations, "
                                 "N(0,0.02^2) bf16 router)",
-        "config": {"workload": f"cfg4 mixed-format MoE decode layer: 512 experts x (2048<->512) SwiGLU, top-10, batch {args.batch}",
+        "config": {"workload": f"cfg4 mixed-format MoE decode layer: 512 experts x (2048<->512) SwiGLU, top-10, batch {args.batch}; "
+                               "weights are random codes in the runtime packed layout (same bytes per expert as packed weights)",
                    "batch": args.batch, "experts": EXPERTS, "hidden": HIDDEN, "intermediate": INTER, "top_k": TOP_K,
                    "format_mix": "NINT2 .10 NINT3 .25 NINT4 .30 NINT8 .05 NVQ3J-L .20 MXFP4 .10",
                    "rotation": f"{work['batches']} token batches x {work['layers']} layer copies",
@@ -329,6 +358,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "moe_rows_fast_kernel<64, true, 16> (gate+up stage)", "achieved": gu_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gu_gbs / HBM_PEAK_GBS,
                      "traffic": measured_traffic(args.batch),
+                     "traffic_source": "profiles/moe_rows_fast_cfg4_b16_pmc.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, "
+                                       "not read in this run)",
                      "bytes_per_launch": gu_bytes, "ms_per_launch": stages["gate_up"],
                      "method": "HIP events recorded by the library on the launch stream around each stage, eager pass "
                                "of the same steps after the timed graph replay",
@@ -349,6 +380,16 @@ def main():
             extra[f"decode_b{b}"] = {"ms_per_step": m, "tok_per_s": b / (m / 1e3), "touched_bytes": tb,
                                      "packed_weight_GBps": tb / (m / 1e3) / 1e9,
                                      "packed_weight_frac_hbm": tb / (m / 1e3) / 1e9 / HBM_PEAK_GBS, "stages_ms": st}
+            del w
+            torch.cuda.empty_cache()
+        for b in (1, 4, 16):
+            w = decode_workload(b, args.steps, args.warmup, args.launch_mode, uniform="NINT4")
+            m = time_graph(w["step"], args.steps, args.warmup)
+            st, tb, dx = stage_profile(w, min(args.steps, 16))
+            extra[f"cfg3_nint4_b{b}"] = {"workload": "cfg3 uniform NINT4 (24-column groups) MoE decode layer, 512 experts, top-10",
+                                         "ms_per_step": m, "tok_per_s": b / (m / 1e3), "touched_bytes": tb,
+                                         "packed_weight_GBps": tb / (m / 1e3) / 1e9,
+                                         "packed_weight_frac_hbm": tb / (m / 1e3) / 1e9 / HBM_PEAK_GBS, "stages_ms": st}
             del w
             torch.cuda.empty_cache()
         extra["prefill_4096"] = prefill_measure()

@@ -117,7 +117,50 @@ def ref_lib():
         R.ref_scaled_i8_dot.argtypes = [_i8p, _f32p, C.c_int, C.c_float, C.c_int]
         R.ref_has_avx2.restype = C.c_int
         R.ref_pool_participants.restype = C.c_int
+        if hasattr(R, "ref_layer"):
+            R.ref_layer.restype = C.c_int
+            R.ref_layer.argtypes = [C.POINTER(_Projection), _i32p, _i32p, C.c_int, _f32p, C.c_int64, C.c_int64, C.c_int,
+                                    C.POINTER(_LayerFns), _f32p]
     return _ref
+
+
+class _LayerFns(C.Structure):
+    """``ref_layer_fns`` of ref_shim.cpp: the pieces of a layer the reference's CPU library does not hold."""
+    _fields_ = [("mx_rows", C.c_void_p), ("swiglu", C.c_void_p), ("f32_to_f16", C.c_void_p), ("f16_to_f32", C.c_void_p),
+                ("nvq_multiplier", C.c_void_p), ("nvq_bank", C.c_void_p)]
+
+
+class RefLayer:
+    """One routed MoE layer prepared for ref_layer(): a single C call runs every routed expert of the batch through
+    the reference's CPU rows kernels (NINT, NVQ) and the C restatement (MXFP4 rows, SwiGLU chain)."""
+
+    def __init__(self, layouts_by_expert: dict, tokens_by_expert: dict, x: np.ndarray):
+        experts = sorted(tokens_by_expert)
+        self._keep = [tuple(Projection(L) for L in layouts_by_expert[e]) for e in experts]
+        self.projections = (_Projection * (3 * len(experts)))()
+        for i, triple in enumerate(self._keep):
+            for j, proj in enumerate(triple):
+                self.projections[3 * i + j] = proj.struct
+        counts = [len(tokens_by_expert[e]) for e in experts]
+        self.offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+        self.token_ids = np.concatenate([np.asarray(tokens_by_expert[e], dtype=np.int32) for e in experts]).astype(np.int32)
+        self.x = np.ascontiguousarray(x, dtype=np.float32)
+        self.hidden = int(self.x.shape[1])
+        self.inter = int(self._keep[0][0].outputs)
+        self.experts = len(experts)
+        self.out = np.zeros((int(self.offsets[-1]), self.hidden), dtype=np.float32)
+        L = lib()
+        self.fns = _LayerFns(*[C.cast(getattr(L, name), C.c_void_p).value for name in
+                               ("orc_mxfp4_rows", "orc_swiglu_array", "orc_f32_to_f16", "orc_f16_to_f32",
+                                "orc_nvq_multiplier", "orc_nvq_bank")])
+
+    def run(self, pooled: bool) -> np.ndarray:
+        status = ref_lib().ref_layer(self.projections, _ptr(self.offsets, _i32p), _ptr(self.token_ids, _i32p), self.experts,
+                                     _ptr(self.x, _f32p), self.hidden, self.inter, int(pooled), C.byref(self.fns),
+                                     _ptr(self.out, _f32p))
+        if status:
+            raise RuntimeError("the reference has no fused rows kernel for one of the formats on this host")
+        return self.out
 
 
 # ------------------------------------------------------------------------------

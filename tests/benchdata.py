@@ -19,11 +19,11 @@ import math
 import numpy as np
 import torch
 
-from . import _lib as L
-from .formats.nint import NintSpec
-from .formats.nvq import NVQ3_D4, NVQ3_D4_1024, codebook_for, pack_jsc_tables
-from .quantize.nvq_quant import initial_jsc_tables
-from .synth import NINT_SPECS, tensor_seed
+from mfq_amd import _lib as L
+from mfq_amd.formats.nint import NintSpec
+from mfq_amd.formats.nvq import NVQ3_D4, NVQ3_D4_1024, codebook_for, pack_jsc_tables
+from mfq_amd.quantize.nvq_quant import initial_jsc_tables
+from synth import NINT_SPECS, tensor_seed
 
 
 class DevicePool:

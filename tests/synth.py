@@ -1,4 +1,5 @@
-"""Synthetic workloads of the benchmark configurations.
+"""Synthetic workloads of the benchmark configurations (used by the tests, bench.py and the smoke run; not part of the
+library).
 
 Random numbers come from a counter-based generator that is trivial to restate in any
 language: ``splitmix64`` of ``seed + counter`` gives 64 uniform bits; two of them feed a
@@ -18,11 +19,11 @@ import math
 
 import numpy as np
 
-from .formats.mfe import MfePool, MfeTensor
-from .formats.mx import Mxfp4Tensor, quantize_mxfp4
-from .formats.nint import NINT2, NINT3, NINT4, NINT8, NintSpec, NintTensor
-from .formats.nvq import NVQ2_E8_4096, NVQ3_D4, NVQ3_D4_1024, NvqJscTensor, NvqTensor
-from .quantize import nint_quant, nvq_quant
+from mfq_amd.formats.mfe import MfePool, MfeTensor
+from mfq_amd.formats.mx import Mxfp4Tensor, quantize_mxfp4
+from mfq_amd.formats.nint import NINT2, NINT3, NINT4, NINT8, NintSpec, NintTensor
+from mfq_amd.formats.nvq import NVQ2_E8_4096, NVQ3_D4, NVQ3_D4_1024, NvqJscTensor, NvqTensor
+from mfq_amd.quantize import nint_quant, nvq_quant
 
 BASE_SEED = 20261125
 _MASK = (1 << 64) - 1

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 from helpers import oracle_layer, rel_l2
-from mfq_amd import synth
+import synth
 from mfq_amd.formats import mfe as MFE, mx, nint, nvq
 from mfq_amd.quantize import nint_quant, nvq_quant
 from oracle import oracle as O

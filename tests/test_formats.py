@@ -9,7 +9,7 @@ import hashlib
 import numpy as np
 import pytest
 
-from mfq_amd import synth
+import synth
 from mfq_amd.formats import bits, mfe as MFE, mx, nint, nvq
 from mfq_amd.quantize import nint_quant, nvq_quant
 

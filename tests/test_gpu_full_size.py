@@ -1,6 +1,6 @@
 """The benchmark's own layers at full size (512 experts x (2048 <-> 512), top-10, mixed formats) through the C ABI.
 
-The weights are the random packed pools of mfq_amd.benchdata, built in device memory; the oracle reads the
+The weights are the random packed pools of tests/benchdata.py, built in device memory; the oracle reads the
 experts a check needs back from the device (runtime layout, one expert at a time), so the CPU side stays at a few
 seconds.  Checks: the decode batch against the oracle end to end (ids bit-exact, output rel-L2 <= 1e-3), sampled
 tokens of the 4096-token prefill against the oracle, and two properties that do not depend on size: doubling the
@@ -24,7 +24,8 @@ _STATE = {}
 def _layer():
     """One full-size mixed-format layer, shared by the tests of this file."""
     if "layer" not in _STATE:
-        from mfq_amd import benchdata, synth
+        import benchdata
+        import synth
         formats = [synth.draw_formats(f"cfg4/format/{p}", EXPERTS) for p in ("gate", "up", "down")]
         _STATE["layer"] = benchdata.device_layer("test/full/layer", EXPERTS, HIDDEN, INTER, formats)
     return _STATE["layer"]
@@ -42,7 +43,8 @@ def _oracle_projections(layer):
 
 def _decode_inputs(tokens):
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     x = synth.to_bf16(synth.normal(f"test/full/x/{tokens}", (tokens, HIDDEN)))
     router = synth.to_bf16(synth.normal("test/full/router", (EXPERTS, HIDDEN), 0.02))
     xd = torch.from_numpy(x).to(torch.bfloat16).cuda()
@@ -67,7 +69,8 @@ def test_decode_batch16_vs_oracle():
 
 def test_prefill_4096_sampled_tokens_vs_oracle():
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     layer = _layer()
     tokens = 4096
     x = synth.to_bf16(synth.normal("test/full/prefill/x", (tokens, HIDDEN)))

@@ -17,7 +17,8 @@ _LAYERS = {}
 
 
 def _layer(tag, experts, hidden, inter, mode, mix=ALL_FORMATS, uniform=None):
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     key = (tag, experts, hidden, inter, mode, uniform)
     if key not in _LAYERS:
         tensors, formats = synth.build_layer(tag, experts, hidden, inter, mix=mix, mode=mode, uniform=uniform)
@@ -26,7 +27,7 @@ def _layer(tag, experts, hidden, inter, mode, mix=ALL_FORMATS, uniform=None):
 
 
 def _inputs(tag, tokens, experts, hidden, k):
-    from mfq_amd import synth
+    import synth
     x = synth.to_bf16(synth.normal(f"{tag}/x", (tokens, hidden)))
     router = synth.to_bf16(synth.normal(f"{tag}/router", (experts, hidden), 0.02))
     logits = O.router_logits(x, router)
@@ -161,7 +162,8 @@ def test_many_pairs_per_expert_and_large_activations():
     the fp16 stage outputs of the reference chain itself, smaller ones push the hidden values into
     fp16 subnormals where one rounding flips whole percents)."""
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     experts, hidden, inter, k, tokens = 6, 256, 64, 3, 32
     tensors, runtimes, _ = _layer("test/moe/few", experts, hidden, inter, "random")
     x, ids, weights = _inputs("test/moe/few/in", tokens, experts, hidden, k)
@@ -203,7 +205,8 @@ def test_layer_with_fused_routing_equals_topk_then_layer(tokens, experts, k):
 def test_layer_with_the_router_matmul_in_front(tokens):
     """run_router = router matmul + top-k + layer in one call: same routes and output as the three calls."""
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     experts, hidden, inter, k = 24, 512, 128, 6
     tensors, runtimes, _ = _layer("test/moe/random", experts, hidden, inter, "random")
     x = synth.to_bf16(synth.normal(f"test/moe/router/x/{tokens}", (tokens, hidden)))
@@ -264,7 +267,8 @@ def test_decode_layer_replayed_from_a_hip_graph():
 def test_prefill_ffn_vs_oracle(tokens):
     """More tokens than the decode limit: route tiles through the MFMA grouped GEMM."""
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     experts, hidden, inter, k = 24, 512, 128, 6
     tensors, runtimes, _ = _layer("test/moe/random", experts, hidden, inter, "random")
     x = synth.to_bf16(synth.normal(f"test/prefill/x/{tokens}", (tokens, hidden)))
@@ -289,7 +293,8 @@ def test_prefill_ffn_vs_oracle(tokens):
 ])
 def test_prefill_shapes_vs_oracle(mode, hidden, inter, tokens, experts, k):
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     tensors, runtimes, _ = _layer(f"test/moe/prefill/{mode}/{hidden}/{inter}/{experts}", experts, hidden, inter, mode)
     x = synth.to_bf16(synth.normal(f"test/prefill/shapes/x/{tokens}/{hidden}", (tokens, hidden)))
     ids = synth.zipf_routes(f"test/prefill/shapes/ids/{tokens}/{experts}", tokens, experts, k)
@@ -307,7 +312,8 @@ def test_prefill_shapes_vs_oracle(mode, hidden, inter, tokens, experts, k):
 def test_prefill_uniform_layer(uniform):
     """Every weight class of the streaming tile kernel on its own, quantised weights with one code width."""
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     experts, hidden, inter, k, tokens = 6, 512, 128, 3, 150
     tensors, runtimes, _ = _layer(f"test/moe/prefill/uniform/{uniform}", experts, hidden, inter, "pack", uniform=uniform)
     x = synth.to_bf16(synth.normal("test/prefill/uniform/x", (tokens, hidden)))
@@ -323,7 +329,8 @@ def test_prefill_uniform_layer(uniform):
 def test_prefill_f16_activations_and_stage_buffers():
     """fp16 activations take the pair shuffle without conversion; gate/up and pair outputs match the oracle stages."""
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     experts, hidden, inter, k, tokens = 12, 512, 128, 4, 90
     tensors, runtimes, _ = _layer("test/moe/prefill/f16", experts, hidden, inter, "random")
     x = synth.normal("test/prefill/f16/x", (tokens, hidden)).astype(np.float16)
@@ -351,7 +358,8 @@ def test_prefill_equals_decode_path():
 def test_grouped_matmul_and_container_reader():
     """MixedMoeRuntime::forward equivalent, with the tensor loaded by the C++ MFE container reader."""
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     from mfq_amd.formats.mfe import pack_mfe
     experts, hidden, inter, k = 12, 256, 64, 4
     tensors, _ = synth.build_layer("test/moe/grouped", experts, hidden, inter, mix=ALL_FORMATS, mode="random")

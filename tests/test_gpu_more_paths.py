@@ -27,7 +27,9 @@ TOL = 1e-3
 ])
 def test_tall_gemv_instantiations_vs_oracle(fmt, rows, width, batch):
     import torch
-    from mfq_amd import _lib as L, benchdata, synth
+    from mfq_amd import _lib as L
+    import benchdata
+    import synth
     print("case", fmt, rows, width, batch, flush=True)
     tensor = benchdata.DeviceMoeTensor(f"test/tall/{fmt}/{rows}/{width}", 1, rows, width, [fmt])
     view = tensor.pools[0].view
@@ -76,7 +78,8 @@ def test_clamped_swiglu_operator_vs_oracle():
 @pytest.mark.parametrize("tokens", [3, 16, 48])     # decode kernels (direct and sorted plans) and the tile kernels
 def test_layer_with_clamped_swiglu_vs_oracle(tokens):
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     from test_gpu_moe import ALL_FORMATS, _inputs, _layer
     experts, hidden, inter, k = 24, 512, 128, 6
     tensors, runtimes, _ = _layer("test/moe/random", experts, hidden, inter, "random")
@@ -99,7 +102,8 @@ def test_dense_single_expert_ffn_feeds_the_shared_gate_epilogue(fmt, tokens):
     """The shared expert: one dense pool per projection (no expert map), every token routed to it with weight 1,
     fp16 output; then out = half(routed + sigmoid(gate) * shared) (mfq/kernels/cuda/moe.cu:1557-1571)."""
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     hidden, inter = (512, 128) if fmt != "NINT3-odd" else (200, 72)      # the odd widths take the exact decoders
     name = "NINT3" if fmt == "NINT3-odd" else fmt
     rng = np.random.default_rng(5)
@@ -131,7 +135,8 @@ def test_layer_with_a_pool_of_per_row_code_widths(tokens):
     """A NINT pool whose rows have different code widths (uniform_bits = 0: the exact decoders read the per-row
     widths and bit offsets) beside streaming pools in one layer."""
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     from mfq_amd.formats import mfe as MFE, nint as FN, nvq as FV
     from mfq_amd.quantize import nint_quant as QN, nvq_quant as QV
     experts, hidden, inter, k = 9, 256, 96, 3
@@ -170,7 +175,9 @@ def test_layer_with_a_pool_of_per_row_code_widths(tokens):
 def test_uniform_nint4_layer_at_full_size_vs_oracle(tokens):
     """512 experts x (2048 <-> 512), every projection NINT4 with 24-column groups, top-10, softmax routing."""
     import torch
-    from mfq_amd import benchdata, runtime as R, synth
+    from mfq_amd import runtime as R
+    import benchdata
+    import synth
     experts, hidden, inter, k = 512, 2048, 512, 10
     if "layer" not in _UNIFORM:
         _UNIFORM["layer"] = benchdata.device_layer("test/cfg3/layer", experts, hidden, inter, [["NINT4"] * experts] * 3)
@@ -204,7 +211,8 @@ def test_token_counts_around_the_largest_decode_plan(tokens):
     """decode_token_limit = 128 with top-10 is clamped to 102 tokens (1020 pairs, one plan thread per pair): 102
     tokens run the decode kernels, more run the grouped GEMM."""
     import torch
-    from mfq_amd import _lib as L, runtime as R, synth
+    from mfq_amd import _lib as L, runtime as R
+    import synth
     from test_gpu_moe import _layer
     experts, hidden, inter, k = 24, 256, 64, 10
     assert L.lib().mfq_amd_moe_ffn_decode_limit(128, k) == 102

@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _router_case(tokens, experts, width, seed):
-    from mfq_amd import synth
+    import synth
     x = synth.to_bf16(synth.normal(f"test/route/x/{seed}", (tokens, width)))
     router = synth.to_bf16(synth.normal(f"test/route/w/{seed}", (experts, width), 0.02))
     return x, router
@@ -77,7 +77,8 @@ def test_topk_half_logits_and_scale():
                                                       (37, 8, 3, 16), (300, 1000, 6, 8), (32, 64, 32, 8), (102, 512, 10, 8), (103, 512, 10, 8)])
 def test_route_plan_matches_oracle(tokens, experts, k, tile_m):
     import torch
-    from mfq_amd import runtime as R, synth
+    from mfq_amd import runtime as R
+    import synth
     if tokens >= 4096:
         ids = synth.zipf_routes("test/plan/zipf", tokens, experts, k)
     else:

@@ -442,3 +442,31 @@ def test_oracle_reproduces_reference_golden_vectors(name):
     assert bits_equal(proj.rows(data["x"], 0), data["y_avx2"])
     if "y_scalar" in data.files:
         assert bits_equal(proj.rows(data["x"], 1), data["y_scalar"])
+
+
+def test_reference_layer_driver_equals_expert_by_expert_rows():
+    """ref_layer (one C call per layer: the CPU baseline of bench.py) gives, pair by pair, what the oracle's expert FFN
+    gives in the reference's summation order, on the calling thread and on the reference's pinned pool."""
+    if O.ref_lib() is None or not hasattr(O.ref_lib(), "ref_layer"):
+        pytest.skip("oracle/_ref not built")
+    rng = np.random.default_rng(33)
+    hidden, inter = 96, 64
+    layouts = {}
+    for e, kinds in enumerate((("nint", "nvq", "mx"), ("nvq", "mx", "nint"), ("mx", "nint", "nvq"))):
+        triple = []
+        for which, kind in enumerate(kinds):
+            rows, width = (inter, hidden) if which < 2 else (hidden, inter)
+            if kind == "nint":
+                triple.append(O.nint_runtime(QN.random_codes(rows, width, FN.NINT4, rng)))
+            elif kind == "nvq":
+                triple.append(O.nvq_runtime(QV.random_nvq_jsc(rows, width, FV.NVQ3_D4_1024, rng)))
+            else:
+                triple.append(O.mxfp4_runtime(FM.random_mxfp4(rows, width, rng)))
+        layouts[e] = tuple(triple)
+    x = rng.normal(0, 1, (5, hidden)).astype(np.float32)
+    tokens = {0: [0, 3], 1: [1, 2, 4], 2: [4]}
+    layer = O.RefLayer(layouts, tokens, x)
+    want = np.concatenate([O.expert_ffn(*[O.Projection(L) for L in layouts[e]], x[tokens[e]], order=0) for e in sorted(tokens)])
+    for pooled in (False, True):
+        got = layer.run(pooled).copy()
+        assert bits_equal(got, want), pooled

@@ -30,7 +30,8 @@ def _run(lib, L, tensor, x, ids, static):
 
 def test_static_scratch_entry_point_matches_the_workspace_entry_point():
     import torch
-    from mfq_amd import _lib as L, runtime as R, synth
+    from mfq_amd import _lib as L, runtime as R
+    import synth
     from helpers import OracleMoeTensor, rel_l2
     lib = L.lib()
     L.check(lib.mfq_amd_init())
@@ -59,7 +60,8 @@ def test_static_scratch_entry_point_matches_the_workspace_entry_point():
 
 def test_static_scratch_entry_point_rejects_what_does_not_fit():
     import torch
-    from mfq_amd import _lib as L, runtime as R, synth
+    from mfq_amd import _lib as L, runtime as R
+    import synth
     lib = L.lib()
     L.check(lib.mfq_amd_init())
     tensors, _ = synth.build_layer("test/static/small", 8, 64, 32, mix=(("NINT4", 1.0),), mode="random")
