@@ -24,6 +24,7 @@
 #pragma once
 
 #include "decode.cuh"
+#include "fetch_at.h"
 
 #include <type_traits>
 
@@ -40,7 +41,6 @@ typedef u32x4 __attribute__((aligned(1))) u32x4_u;
 typedef uint16_t __attribute__((aligned(1))) unaligned_u16;
 
 constexpr uint32_t kMagicPair = 0x64006400u;   // two halves of 1024.0
-constexpr int kLaneColumns = 32;
 
 __device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w), __builtin_bit_cast(half2_t, x), acc, false);
@@ -188,32 +188,6 @@ __device__ constexpr float pair_scale(int k) {
     return 1.0f;
 }
 
-// Per-lane constants of one lane block.
-struct LaneBlock {
-    int cb;            // index of the block in the row, clamped to a valid one
-    bool valid;        // the block lies inside the row
-    uint32_t sel;      // bit j: chunk j of the block belongs to the lane's second group
-    int group;         // first group of the block
-    int level_at;      // NINT: group index at which the 16-bit level window is loaded
-    int level_shift;   //       and the shift that brings the block's first level to bit 0
-};
-
-template <int GS>
-__device__ __forceinline__ LaneBlock lane_block(int cb, int width, int groups) {
-    LaneBlock b;
-    b.valid = cb * kLaneColumns < width;
-    b.cb = b.valid ? cb : 0;
-    b.group = (b.cb * kLaneColumns) / GS;
-    b.sel = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-        if ((b.cb * kLaneColumns + 8 * j) / GS != b.group) b.sel |= 1u << j;
-    // two consecutive levels come with one 16-bit load; the window slides back at the last group
-    b.level_at = b.group < groups - 2 ? b.group : groups - 2;
-    b.level_shift = 8 * (b.group - b.level_at);
-    return b;
-}
-
 // Scale 2^-e that brings `largest` (>= 0) into [2^14, 2^15), and its inverse.
 __device__ __forceinline__ void normaliser(float largest, float& down, float& up) {
     int e = static_cast<int>((__float_as_uint(largest) >> 23) & 0xffu) - 127 - 14;
@@ -338,19 +312,13 @@ __device__ __forceinline__ FastCtx<CLS> fast_ctx(const mfq_amd_projection& p, in
         c.entries = nvq_format_entries(p.format);
         c.nvec8 = p.nvec / 8;
         c.nsign4 = p.nsign / 4;
-        const int64_t index_byte = first_row * c.nvec8 * c.index_bits;
-        const int64_t sign_bit = first_row * c.nsign4 * 28;
-        const int64_t state_bit = first_row * p.groups * 4;
-        c.f0 = static_cast<const uint8_t*>(p.fields[0]) + index_byte;
-        c.f1 = static_cast<const uint8_t*>(p.fields[1]) + (sign_bit >> 3);
-        c.f2 = static_cast<const uint8_t*>(p.fields[2]) + (state_bit >> 3);
+        const NvqExpertAt at = nvq_expert_at(first_row, c.nvec8, c.index_bits, c.nsign4, p.groups, p.sizes[0], p.sizes[1], p.sizes[2]);
+        c.f0 = static_cast<const uint8_t*>(p.fields[0]) + at.index_byte;
+        c.f1 = static_cast<const uint8_t*>(p.fields[1]) + at.sign_byte;
+        c.f2 = static_cast<const uint8_t*>(p.fields[2]) + at.state_byte;
         c.f3 = static_cast<const float*>(p.fields[3]) + first_row;
-        const int64_t left0 = p.sizes[0] - index_byte, left1 = p.sizes[1] - (sign_bit >> 3), left2 = p.sizes[2] - (state_bit >> 3);
-        c.limit0 = static_cast<int>(left0 < 0x7fffffff ? left0 : 0x7fffffff);
-        c.limit1 = static_cast<int>(left1 < 0x7fffffff ? left1 : 0x7fffffff);
-        c.limit2 = static_cast<int>(left2 < 0x7fffffff ? left2 : 0x7fffffff);
-        c.sign_bit0 = static_cast<int>(sign_bit & 7);
-        c.state_bit0 = static_cast<int>(state_bit & 7);
+        c.limit0 = at.limit0; c.limit1 = at.limit1; c.limit2 = at.limit2;
+        c.sign_bit0 = at.sign_bit0; c.state_bit0 = at.state_bit0;
         c.multiplier = reinterpret_cast<const float*>(lds);
         c.bank_byte = reinterpret_cast<const int*>(lds + 64);
         c.signs = lds + 128;
@@ -387,51 +355,38 @@ __device__ __forceinline__ FastRaw<CLS> fast_fetch(const FastCtx<CLS>& c, const 
     using C = FastClass<CLS>;
     FastRaw<CLS> raw{};
     if constexpr (C::kNint) {
-        // the row part of every address first: it is the same in all lanes when a wave works on one row,
-        // and then stays in scalar registers
-        load_dwords<C::kQ>(c.f0 + static_cast<uint32_t>(row) * c.row_bytes + static_cast<uint32_t>(b.cb * (4 * C::kBits)), raw.q);
+        // (the row part of every address is the same in all lanes when a wave works on one row, and then stays in
+        // scalar registers)
+        const NintFetchAt at = nint_fetch_at(row, c.row_bytes, c.groups, C::kBits, C::kGs, b);
+        load_dwords<C::kQ>(c.f0 + at.code_byte, raw.q);
         if constexpr (LEVELS) {
-            const uint8_t* scale_row = c.f1 + static_cast<uint32_t>(row) * c.groups;
-            const uint8_t* min_row = c.f2 + static_cast<uint32_t>(row) * c.groups;
             if constexpr (C::kGs == 32) {
-                raw.a = gload<uint8_t>(scale_row + static_cast<uint32_t>(b.group));
-                raw.b = gload<uint8_t>(min_row + static_cast<uint32_t>(b.group));
+                raw.a = gload<uint8_t>(c.f1 + at.level_byte);
+                raw.b = gload<uint8_t>(c.f2 + at.level_byte);
             } else {
-                raw.a = *(const MFQ_GLOBAL unaligned_u16*)(scale_row + static_cast<uint32_t>(b.level_at));
-                raw.b = *(const MFQ_GLOBAL unaligned_u16*)(min_row + static_cast<uint32_t>(b.level_at));
+                raw.a = *(const MFQ_GLOBAL unaligned_u16*)(c.f1 + at.level_byte);
+                raw.b = *(const MFQ_GLOBAL unaligned_u16*)(c.f2 + at.level_byte);
             }
         }
     } else if constexpr (C::kMx) {
-        load_dwords<4>(c.f0 + static_cast<uint32_t>(row) * c.row_bytes + static_cast<uint32_t>(b.cb * 16), raw.q);
-        if constexpr (LEVELS) raw.a = gload<uint8_t>(c.f1 + static_cast<uint32_t>(row) * (c.row_bytes / 16) + static_cast<uint32_t>(b.cb));
+        const MxFetchAt at = mx_fetch_at(row, c.row_bytes, b);
+        load_dwords<4>(c.f0 + at.code_byte, raw.q);
+        if constexpr (LEVELS) raw.a = gload<uint8_t>(c.f1 + at.scale_byte);
     } else {
-        // Every offset is a row part plus a lane part; the row part is the same in all lanes when a wave
-        // works on one row, and written apart it stays in scalar registers.
+        const NvqFetchAt at = nvq_fetch_at(row, c.nvec8, c.index_bits, c.nsign4, c.groups, c.limit0, c.limit2, c.sign_bit0,
+                                           c.state_bit0, b);
         // eight indices: index_bits bytes, byte aligned because a row holds a multiple of 8 vectors
-        const uint32_t index_byte = static_cast<uint32_t>(row) * static_cast<uint32_t>(c.nvec8 * c.index_bits) +
-                                    static_cast<uint32_t>(b.cb * c.index_bits);
-        const u32x2 lo = *(const MFQ_GLOBAL u32x2_u*)(c.f0 + index_byte);
+        const u32x2 lo = *(const MFQ_GLOBAL u32x2_u*)(c.f0 + at.index_byte);
         raw.q[0] = lo[0]; raw.q[1] = lo[1];
-        const int wanted = static_cast<int>(index_byte) + 8;
-        const int third = wanted < c.limit0 - 4 ? wanted : c.limit0 - 4;
-        raw.q[2] = load_u32_unaligned(c.f0 + third);
+        raw.q[2] = load_u32_unaligned(c.f0 + at.third_byte);
         if constexpr (LEVELS) {
-            // four 7-bit sign masks: 28 bits that start on a nibble boundary, always inside one dword
-            const uint32_t sign_bit = static_cast<uint32_t>(row) * static_cast<uint32_t>(c.nsign4 * 28) +
-                                      static_cast<uint32_t>(b.cb * 28 + c.sign_bit0);
-            raw.a = load_u32_unaligned(c.f1 + (sign_bit >> 3));
-            // the states of the block's two groups
-            const uint32_t state_bit = static_cast<uint32_t>(row) * static_cast<uint32_t>(c.groups * 4) +
-                                       static_cast<uint32_t>(b.group * 4 + c.state_bit0);
-            const int state_byte = static_cast<int>(state_bit >> 3);
-            const int at = state_byte < c.limit2 - 2 ? state_byte : c.limit2 - 2;
-            raw.c = *(const MFQ_GLOBAL unaligned_u16*)(c.f2 + at);
+            raw.a = load_u32_unaligned(c.f1 + at.sign_byte);     // four 7-bit sign masks
+            raw.c = *(const MFQ_GLOBAL unaligned_u16*)(c.f2 + at.state_byte);   // the states of the block's two groups
             // shifts that bring the three loaded words into place; applied when the data is consumed so that
             // nothing here waits for a load
-            raw.b = ((8u * static_cast<uint32_t>(wanted - third)) & 31u) | ((sign_bit & 7u) << 8) |
-                    (((state_bit & 7u) + 8u * static_cast<uint32_t>(state_byte - at)) << 16);
+            raw.b = at.shifts;
         } else {
-            raw.b = (8u * static_cast<uint32_t>(wanted - third)) & 31u;
+            raw.b = at.shifts & 0xffu;
         }
     }
     return raw;

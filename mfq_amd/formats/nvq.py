@@ -294,29 +294,33 @@ def pack_jsc_group64(state: np.ndarray, indices: np.ndarray, signs: np.ndarray, 
     return np.ascontiguousarray(records, dtype="<u8").tobytes()
 
 
+def _field(planes: np.ndarray, first: int, width: int) -> np.ndarray:
+    """Bits [first, first + width) of every record as integers; ``planes`` holds one bit per column, LSB first."""
+    weights = (1 << np.arange(width, dtype=np.uint32))
+    return planes[..., first:first + width].astype(np.uint32) @ weights
+
+
 def unpack_jsc_group64(blob, off: int, out: int, neuron_len: int):
-    """Inverse of pack_jsc_group64; checks the parity bits and the zero padding (mfq/formats/nvq.py:727-760)."""
+    """Inverse of pack_jsc_group64: the records are read as 64 bit planes (the layout of bits.py: LSB first), from
+    which the state, the three indices, sign masks and parity bits are sliced by position.  Parity bits and the zero
+    padding behind a row's last vector are checked (record layout: mfq/formats/nvq.py:659-716)."""
     groups, vectors = -(-neuron_len // GROUP), -(-neuron_len // 8)
-    if off + out * groups * 8 > len(blob):
+    nbytes = out * groups * 8
+    if off + nbytes > len(blob):
         raise ValueError("truncated NVQ-JSC group64 stream")
-    records = np.frombuffer(blob, dtype="<u8", count=out * groups, offset=off).reshape(out, groups)
-    state = (records >> np.uint64(60)).astype(np.uint8)
-    indices = np.zeros((out, groups * 3), dtype=np.uint16)
-    signs = np.zeros((out, groups * 3), dtype=np.uint8)
-    for local in range(3):
-        segment = (records >> np.uint64(20 * local)) & np.uint64(0xFFFFF)
-        sign8 = (segment >> np.uint64(12)).astype(np.uint8)
-        sign7 = sign8 & np.uint8(0x7F)
-        parity = np.zeros_like(sign7)
-        for bit in range(7):
-            parity ^= (sign7 >> np.uint8(bit)) & np.uint8(1)
-        if np.any((sign8 >> np.uint8(7)) != parity):
-            raise ValueError("invalid NVQ-JSC group64 parity bit")
-        indices[:, local::3] = (segment & np.uint64(0xFFF)).astype(np.uint16)
-        signs[:, local::3] = sign7
-    if np.any(indices[:, vectors:]) or np.any(signs[:, vectors:]):
+    raw = np.frombuffer(blob, dtype=np.uint8, count=nbytes, offset=off)
+    planes = np.unpackbits(raw, bitorder="little").reshape(out, groups, 64)
+    state = _field(planes, 60, 4).astype(np.uint8)
+    # segment s of a record covers bits [20 s, 20 s + 20): index (12), sign mask (7), parity of the mask (1)
+    segments = planes[..., :60].reshape(out, groups * 3, 20)
+    masks = segments[..., 12:19]
+    if np.any(segments[..., 19] != (masks.sum(axis=-1) & 1)):
+        raise ValueError("invalid NVQ-JSC group64 parity bit")
+    if np.any(segments[:, vectors:, :]):
         raise ValueError("NVQ-JSC group64 padding must be zero")
-    return state, indices[:, :vectors].copy(), signs[:, :vectors].copy(), off + out * groups * 8
+    indices = _field(segments[:, :vectors], 0, 12).astype(np.uint16)
+    signs = _field(segments[:, :vectors], 12, 7).astype(np.uint8)
+    return state, indices, signs, off + nbytes
 
 
 def pack_jsc_tables(scale_lut: np.ndarray, bank_for_state: np.ndarray, codebooks: np.ndarray,

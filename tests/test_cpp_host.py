@@ -94,3 +94,20 @@ def test_cpp_ffn_equals_the_python_mirror_and_the_oracle(tmp_path, tokens):
     runtimes = [R.MixedMoeRuntime.from_blob(blob) for blob in blobs]
     mirror = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens).run_logits(xd, logits).cpu().numpy()
     assert np.array_equal(fused.view(np.uint32), mirror.view(np.uint32))
+
+
+def test_streaming_fetches_stay_inside_their_fields(tmp_path):
+    """The address arithmetic the streaming kernels run on the device (mfq_amd/csrc/fetch_at.h), compiled for the host
+    and swept over every kernel class, widths from 32 to 4096, 1..70 rows and up to three experts per pool: no fetch
+    reads a byte outside the packed field it reads from (including the NVQ sign-mask load, which is not clamped)."""
+    import shutil
+    import subprocess
+    compiler = shutil.which("g++") or shutil.which("hipcc")
+    if compiler is None:
+        pytest.skip("no host C++ compiler")
+    binary = tmp_path / "fetch_extent_check"
+    source = ROOT / "tests" / "cpp" / "fetch_extent_check.cpp"
+    subprocess.run([compiler, "-O2", "-std=c++17", str(source), "-o", str(binary)], check=True)
+    done = subprocess.run([str(binary)], capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
+    assert "fetches inside their fields" in done.stdout and int(done.stdout.split()[0]) > 1_000_000
