@@ -209,15 +209,17 @@ def cpu_baseline(work, samples=7, budget_s=25.0):
                                "the SwiGLU chain through the C restatement; median"}
 
 
-def prefill_measure(tokens=4096, reps=7):
+def prefill_measure(tokens=4096, reps=7, uniform=None, mx_scaled=False):
+    """uniform: one format for every projection instead of the drawn mix; mx_scaled: MXFP4 tiles on the block-scaled
+    MFMA with the activations split into E4M3 terms (the split runs inside the timed gate/up and down stages)."""
     import numpy as np
     import torch
     from mfq_amd import runtime as R
     import benchdata
     import synth
-    formats = [synth.draw_formats(f"cfg4/format/{p}", EXPERTS) for p in ("gate", "up", "down")]
-    layer = benchdata.device_layer("cfg5/layer", EXPERTS, HIDDEN, INTER, formats)
-    ffn = R.MfeFfnRuntime(*layer, top_k=TOP_K, max_tokens=tokens)
+    formats = [[uniform] * EXPERTS if uniform else synth.draw_formats(f"cfg4/format/{p}", EXPERTS) for p in ("gate", "up", "down")]
+    layer = benchdata.device_layer(f"cfg5/{uniform}" if uniform else "cfg5/layer", EXPERTS, HIDDEN, INTER, formats)
+    ffn = R.MfeFfnRuntime(*layer, top_k=TOP_K, max_tokens=tokens, mx_scaled_mfma=mx_scaled)
     x = torch.from_numpy(synth.to_bf16(synth.normal("cfg5/x", (tokens, HIDDEN)))).to(torch.bfloat16).cuda()
     ids = torch.from_numpy(synth.zipf_routes("cfg5/zipf", tokens, EXPERTS, TOP_K)).cuda()
     w = torch.full((tokens, TOP_K), 1.0 / TOP_K, dtype=torch.float32, device="cuda")
@@ -236,7 +238,9 @@ def prefill_measure(tokens=4096, reps=7):
     total_ms = sum(best.values())
     return {"tokens": tokens, "ms_layer": total_ms, "ms_gemm": gemm_ms, "tok_per_s": tokens / (total_ms / 1e3),
             "tflops_gemm": flops / (gemm_ms / 1e3) / 1e12, "mfma_frac_of_f16_peak": flops / (gemm_ms / 1e3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
-            "stages_ms": best, "element_type": "fp16 tiles, fp32 accumulate", "samples": reps, "statistic": "median run"}
+            "stages_ms": best, "samples": reps, "statistic": "median run",
+            "element_type": "E4M3 activation terms x E2M1 weights on the block-scaled MFMA, fp32 accumulate" if mx_scaled
+                            else "fp16 tiles, fp32 accumulate"}
 
 
 def gemv_measure(calls=64):
@@ -323,7 +327,9 @@ def main():
         sys.exit(2)
     torch.cuda.set_device(0)
     if args.prefill_only:
-        print(json.dumps({"prefill_4096": prefill_measure()}))
+        print(json.dumps({"prefill_4096": prefill_measure(),
+                          "prefill_4096_mxfp4_f16_tiles": prefill_measure(uniform="MXFP4"),
+                          "prefill_4096_mxfp4_block_scaled": prefill_measure(uniform="MXFP4", mx_scaled=True)}))
         return
 
     work = decode_workload(args.batch, args.steps, args.warmup, args.launch_mode)

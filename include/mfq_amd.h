@@ -198,7 +198,11 @@ typedef struct mfq_amd_moe_ffn_config {
                                 * (mfq_amd_moe_ffn_decode_limit gives the value create will use). */
     int32_t launch_mode;       /* decode: 0 = one launch per stage covering every format (blocks sorted by
                                   format), 1 = one launch per format and stage */
-    int32_t reserved[3];
+    int32_t mx_scaled_mfma;    /* 1: prefill tiles of MXFP4 pools run on the block-scaled MFMA (v_mfma_scale_f32_32x32x64_f8f6f4:
+                                  fp4 weights with their E8M0 scales as stored, activations as E4M3 terms that add up to the
+                                  source exactly); 0: on the fp16 tiles like every other format.  Counterpart of
+                                  mxfp4_moe_grouped_tensor_kernel (mfq/kernels/cuda/mx_matmul.cu:954). */
+    int32_t reserved[2];
 } mfq_amd_moe_ffn_config;
 
 /* create may allocate and synchronise; run allocates nothing, does not synchronise and can be

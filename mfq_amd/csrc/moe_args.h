@@ -32,6 +32,10 @@ struct RowsArgs {
     int64_t in_packed_stride;          // dwords between packed rows
     const uint16_t* in_tiles;          // the same rows as fp16 in the pair order of the weight classes (tile kernel), or null
     int64_t in_tiles_layout_stride;    // halves between the copies in the four pair layouts; 0: rows are in the order their consumer needs
+    const uint8_t* in_fp8;             // block-scaled MFMA kernel: the activation rows as E4M3 terms, [row][terms][in_width] bytes
+    const uint8_t* in_fp8_scales;      // their E8M0 block scales, [row][terms][in_width / 32]
+    int32_t in_fp8_terms;              // 2 (bf16 source) or 3 (fp16 source): the terms add up to the source exactly
+    int32_t skip_mxfp4;                // streaming tile kernel: leave MXFP4 tiles to the block-scaled MFMA kernel
     const uint16_t* gu;                // streaming decode kernel, down projection: gate/up outputs f16 [pair][2][in_width]; the block
                                        // computes hidden = swiglu(gate, up) of its pair itself.  Null: activations come from in / in_packed
     const uint16_t* sigmoid;           // the sigmoid table swiglu uses (gu != null)
@@ -67,6 +71,12 @@ bool tiles_fast_geometry(int in_width, int in_dtype, int in_vector_ok);
 // Streaming MFMA tile kernel, one launch for every class; max_tiles bounds the tiles of a slot.
 // Tiles of pools marked kPoolExactOnly are skipped.
 void launch_tiles_fast(const RowsArgs& args, int slots, int max_tiles, bool nvq, hipStream_t stream);
+// MXFP4 tiles on the block-scaled MFMA of gfx950 (fp4 weights with their E8M0 scales straight from memory, activations as
+// E4M3 terms): the tiles of class K_MXFP4 of the plan; other tiles are skipped.
+void launch_tiles_mx_scaled(const RowsArgs& args, int slots, int max_tiles, hipStream_t stream);
+// dst[row][terms][width] E4M3 bytes and scales[row][terms][width / 32] E8M0 bytes of src[row][width] (fp16 or bf16);
+// the terms of a block add up to the source values exactly (2 terms for bf16, 3 for fp16).
+void launch_fp8_split(const void* src, int dtype, int rows, int width, int terms, uint8_t* dst, uint8_t* scales, hipStream_t stream);
 // Pair layout (0..3) in which the streaming tile kernel reads the activations of a pool of this class.
 int tile_layout_of_class(int cls);
 // dst[layout][rows][width] = fp16 copy of src (fp16 or bf16) in the pair order of every layout in the mask.

@@ -8,6 +8,7 @@
 #include "launch.cuh"
 #include "moe_args.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -597,6 +598,8 @@ struct mfq_amd_moe_ffn {
     int32_t* d_route_ids = nullptr;      // routes selected by run_logits
     float* d_route_weights = nullptr;
     uint32_t *d_x_packed = nullptr, *d_hidden_packed = nullptr;
+    uint8_t *d_fp8 = nullptr, *d_fp8_scales = nullptr;   // prefill, block-scaled MFMA: activations as E4M3 terms and their block scales
+    bool mx_scaled[kSlots] = {false, false, false};      // the slot has MXFP4 pools that run on the block-scaled MFMA
     uint16_t* d_x_tiles = nullptr;       // prefill: fp16 copies of the token rows in the pair layouts of the gate/up pools
     uint32_t x_tile_layouts = 0;         // mask of those layouts   // decode only: activations as the streaming kernels read them
     int tile_capacity = 0;
@@ -610,7 +613,7 @@ struct mfq_amd_moe_ffn {
     ~mfq_amd_moe_ffn() {
         void* all[] = {d_pools, d_pool_class, d_pool_bytes, d_expert_pool, d_expert_info, d_expert_words, d_item_info, d_pair_items, d_items, d_class_offsets, d_tile_items,
                        d_tile_offsets, d_counts, d_bounds, d_tile_bounds, d_tile_experts, d_ids_dst, d_distinct,
-                       d_touched, d_gu, d_hidden, d_pairs, d_logits, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base};
+                       d_touched, d_gu, d_hidden, d_pairs, d_logits, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base, d_fp8, d_fp8_scales};
         for (void* p : all) if (p) (void)hipFree(p);
         for (hipEvent_t e : events) if (e) (void)hipEventDestroy(e);
     }
@@ -629,6 +632,7 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
         MFQ_REQUIRE(c.x_dtype >= MFQ_AMD_F32 && c.x_dtype <= MFQ_AMD_BF16, "unknown activation dtype");
         MFQ_REQUIRE(c.out_dtype == MFQ_AMD_F32 || c.out_dtype == MFQ_AMD_F16, "output must be float32 or float16");
         MFQ_REQUIRE(c.launch_mode == 0 || c.launch_mode == 1, "unknown launch mode");
+        MFQ_REQUIRE(c.mx_scaled_mfma == 0 || c.mx_scaled_mfma == 1, "mx_scaled_mfma must be 0 or 1");
         MFQ_REQUIRE(c.gate.experts == c.up.experts && c.gate.experts == c.down.experts, "expert counts differ");
         MFQ_REQUIRE(c.gate.neuron_len == c.up.neuron_len && c.gate.out_per_expert == c.up.out_per_expert &&
                     c.down.neuron_len == c.gate.out_per_expert && c.down.out_per_expert == c.gate.neuron_len,
@@ -718,6 +722,18 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
                 for (int i = f->tables.slot_begin[s]; i < f->tables.slot_begin[s + 1]; ++i)
                     if (!(f->tables.classes[i] & kPoolExactOnly)) f->x_tile_layouts |= 1u << tile_layout_of_class(f->tables.classes[i]);
             if (f->x_tile_layouts) f->d_x_tiles = device_alloc<uint16_t>(static_cast<size_t>(4) * c.max_tokens * f->hidden);
+            if (c.mx_scaled_mfma && c.x_dtype != MFQ_AMD_F32 && tiles_fast_geometry(f->intermediate, MFQ_AMD_F16, 1)) {
+                bool any = false;
+                for (int s = 0; s < kSlots; ++s) {
+                    f->mx_scaled[s] = f->tables.present[s][dev::K_MXFP4] && !f->tables.exact_present[s][dev::K_MXFP4];
+                    any = any || f->mx_scaled[s];
+                }
+                if (any) {
+                    const size_t most = std::max(static_cast<size_t>(c.max_tokens) * f->hidden, static_cast<size_t>(pairs) * f->intermediate) * 3;
+                    f->d_fp8 = device_alloc<uint8_t>(most);
+                    f->d_fp8_scales = device_alloc<uint8_t>(most / dev::kLaneColumns);
+                }
+            }
         }
         {
             bool exact_work = c.launch_mode != 0 || !rows_fast_geometry(f->hidden, c.x_dtype) ||
@@ -833,9 +849,19 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
                 const bool tiles = f->config.launch_mode == 0 && tiles_fast_geometry(rows.in_width, rows.in_dtype, rows.in_vector_ok);
                 if (!tiles) rows.in_tiles = nullptr;
                 if (tiles) {
-                    bool nvq = false;
-                    for (int s = slot_lo; s < slot_hi; ++s) nvq = nvq || f->tables.fast_nvq[s];
+                    bool nvq = false, mx = false;
+                    for (int s = slot_lo; s < slot_hi; ++s) { nvq = nvq || f->tables.fast_nvq[s]; mx = mx || f->mx_scaled[s]; }
+                    mx = mx && f->d_fp8 != nullptr;
+                    if (mx) {
+                        // MXFP4 tiles on the block-scaled MFMA: the activations of the stage as E4M3 terms first
+                        const int terms = rows.in_dtype == MFQ_AMD_BF16 ? 2 : 3;
+                        launch_fp8_split(rows.in, rows.in_dtype, rows.in_per_pair ? pairs : tokens, rows.in_width, terms, f->d_fp8,
+                                         f->d_fp8_scales, stream);
+                        rows.in_fp8 = f->d_fp8; rows.in_fp8_scales = f->d_fp8_scales; rows.in_fp8_terms = terms;
+                    }
+                    rows.skip_mxfp4 = mx ? 1 : 0;
                     launch_tiles_fast(rows, slots, pairs / kPrefillTileM + active_bound, nvq, stream);
+                    if (mx) launch_tiles_mx_scaled(rows, slots, pairs / kPrefillTileM + active_bound, stream);
                 }
                 rows.exact_only = tiles ? 1 : 0;
                 if (class_bounds(slot_lo, slot_hi, true, tiles)) launch_rows_prefill(rows, slots, present, bound, stream);

@@ -16,6 +16,7 @@
 #include "decode.cuh"
 #include "device_state.h"
 #include "fast.cuh"
+#include "fp8_split.h"
 #include "launch.cuh"
 #include "moe_args.h"
 #include "xpack.cuh"
@@ -594,8 +595,178 @@ __global__ void __launch_bounds__(256, 2) moe_tiles_fast_kernel(RowsArgs a) {
         case K_NINT_4_32: tiles_fast_class<K_NINT_4_32, PACKED>(a, slot, row_block, pool, local, begin, count, lds); break;
         case K_NINT_8_48: tiles_fast_class<K_NINT_8_48, PACKED>(a, slot, row_block, pool, local, begin, count, lds); break;
         case K_NVQ_D4: tiles_fast_class<K_NVQ_D4, PACKED>(a, slot, row_block, pool, local, begin, count, lds); break;
-        case K_MXFP4: tiles_fast_class<K_MXFP4, PACKED>(a, slot, row_block, pool, local, begin, count, lds); break;
+        case K_MXFP4: if (!a.skip_mxfp4) tiles_fast_class<K_MXFP4, PACKED>(a, slot, row_block, pool, local, begin, count, lds); break;
         default: break;   // pools marked kPoolExactOnly and classes without a streaming path
+    }
+}
+
+// ------------------------------------------------- MXFP4 on the block-scaled MFMA ----
+// v_mfma_scale_f32_32x32x64_f8f6f4: D[32 x 32] += (A * 2^(sa-127)) (B * 2^(sb-127)) over 64 columns in two blocks of 32,
+// one E8M0 scale per row and block: lanes 0..31 bring the scales of block 0, lanes 32..63 those of block 1.  Where the
+// columns lie depends on the operand's format.  A 4-bit operand has its lane hold the 32 columns of its block (16 bytes,
+// low nibble first), which is the MXFP4 storage itself: 16 bytes of nibbles and one scale byte per 32 columns of a
+// weight row go into B as they lie in memory, no arithmetic.  An 8-bit operand has lane half h hold columns
+// 16 h .. 16 h + 15 of block 0 in its first four registers and the same columns of block 1 in the other four.  The
+// activations come as E4M3 terms (fp8_split.h) that add up to the source exactly, one MFMA per term; fp32 accumulation.
+// A block = one plan tile (up to 128 pairs of one expert) x 256 output rows, a wave 64 of the rows, as in the
+// streaming tile kernel.  Every lane of a wave must be active at the MFMA: lanes switched off read as zero operands.
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+template <int MT, int TERMS>
+__device__ __forceinline__ void tiles_mx_scaled_block(const RowsArgs& a, int slot, int row_block, const mfq_amd_projection& pool, int local,
+                                                      int begin, int count) {
+    const int tid = threadIdx.x, lane = tid % kWave, wave = uniform(static_cast<int>(tid / kWave));
+    const int n = lane & 31, h = lane >> 5;
+    const int width = a.in_width, blocks = width / kLaneColumns;
+    const int steps = (blocks + 1) / 2;
+    const int64_t first_row = static_cast<int64_t>(local) * pool.output_rows;
+    const uint8_t* codes = static_cast<const uint8_t*>(pool.fields[0]) + first_row * (width / 2);
+    const uint8_t* scales = static_cast<const uint8_t*>(pool.fields[1]) + first_row * blocks;
+    // weights: lane -> rows n and n + 32 of the wave's 64
+    const int n0 = row_block * kFastTileN + wave * 64;
+    int rows[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        rows[t] = n0 + 32 * t + n;
+        rows[t] = rows[t] < a.out_rows ? rows[t] : a.out_rows - 1;
+    }
+    // activations: lane -> pair 32 mt + n of the tile (clamped: rows behind the last pair are computed and not stored)
+    const uint8_t* x_rows[MT];
+    const uint8_t* x_scales[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = 32 * mt + n;
+        const int pair = a.ids_dst[begin + (m < count ? m : 0)];
+        const int64_t source = a.in_per_pair ? pair : pair / a.top_k;
+        x_rows[mt] = a.in_fp8 + source * TERMS * width;
+        x_scales[mt] = a.in_fp8_scales + source * TERMS * blocks;
+    }
+    float16_t acc[2][MT];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[t][mt][i] = 0.0f;
+
+    for (int step = 0; step < steps; ++step) {
+        int cb = 2 * step + h;
+        const bool inside = cb < blocks;
+        cb = inside ? cb : blocks - 1;
+        i32x8 b[2];
+        int sb[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const u32x4 q = *(const MFQ_GLOBAL u32x4*)(codes + static_cast<int64_t>(rows[t]) * (width / 2) + cb * 16);
+            // a lane block behind the end of the row (odd block counts) contributes nothing: zero codes
+            b[t] = i32x8{inside ? static_cast<int>(q[0]) : 0, inside ? static_cast<int>(q[1]) : 0, inside ? static_cast<int>(q[2]) : 0,
+                         inside ? static_cast<int>(q[3]) : 0, 0, 0, 0, 0};
+            sb[t] = gload<uint8_t>(scales + static_cast<int64_t>(rows[t]) * blocks + cb);
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+            for (int term = 0; term < TERMS; ++term) {
+                const uint8_t* at = x_rows[mt] + term * width + step * 64 + 16 * h;
+                const u32x4 lo = *(const MFQ_GLOBAL u32x4*)at;
+                u32x4 hi = {0u, 0u, 0u, 0u};                                    // no second block behind an odd count
+                if (2 * step + 1 < blocks) hi = *(const MFQ_GLOBAL u32x4*)(at + 32);
+                const i32x8 av = {static_cast<int>(lo[0]), static_cast<int>(lo[1]), static_cast<int>(lo[2]), static_cast<int>(lo[3]),
+                                  static_cast<int>(hi[0]), static_cast<int>(hi[1]), static_cast<int>(hi[2]), static_cast<int>(hi[3])};
+                const int sa = gload<uint8_t>(x_scales[mt] + term * blocks + cb);
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    acc[t][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, b[t], acc[t][mt], 0 /* A: E4M3 */, 4 /* B: E2M1 */,
+                                                                                   0, sa, 0, sb[t]);
+            }
+        }
+    }
+    // D[m][n]: the lane holds row n of the weights and pairs m = 8 * (i / 4) + 4 * h + i % 4 of each 32
+    uint16_t* out = a.out + (slot - a.slot_base) * a.out_slot_stride;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int row = n0 + 32 * t + n;
+        if (row >= a.out_rows) continue;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int m = 32 * mt + 8 * (i / 4) + 4 * h + (i % 4);
+                if (m < count) out[static_cast<int64_t>(a.ids_dst[begin + m]) * a.out_pair_stride + row] = float_to_half_bits(acc[t][mt][i]);
+            }
+    }
+}
+
+template <int TERMS>
+__global__ void __launch_bounds__(256) moe_tiles_mx_scaled_kernel(RowsArgs a) {
+    // same block -> (tile, row block, slot) order as the streaming tile kernel
+    const int row_blocks = (a.out_rows + kFastTileN - 1) / kFastTileN;
+    const int sharers = row_blocks * a.tile_slots;
+    const int id = blockIdx.x;
+    const int index = id / (8 * sharers) * 8 + id % 8;
+    const int sub = id % (8 * sharers) / 8;
+    const int row_block = sub / a.tile_slots;
+    const int slot = a.slot_base + sub % a.tile_slots;
+    const int* offsets = a.tile_offsets + slot * kClassSlots;
+    // tile_items is sorted by class: only the MXFP4 range concerns this kernel
+    if (index < offsets[K_MXFP4] || index >= offsets[K_MXFP4 + 1] || index >= a.tile_capacity) return;
+    const int packed = a.tile_items[slot * a.tile_capacity + index];
+    const int expert = packed & 0xffff, m_tile = packed >> 16;
+    const ExpertInfo info = a.expert_info[slot * a.experts + expert];
+    if (info.pool < 0 || info.cls != K_MXFP4) return;
+    const int begin = a.expert_bounds[expert] + m_tile * kPrefillTileM;
+    const int left = a.expert_bounds[expert + 1] - begin;
+    const int count = left < kPrefillTileM ? left : kPrefillTileM;
+    if (count <= 0) return;
+    const mfq_amd_projection& pool = a.pools[info.pool];
+    if (count <= 32) tiles_mx_scaled_block<1, TERMS>(a, slot, row_block, pool, info.local, begin, count);
+    else if (count <= 64) tiles_mx_scaled_block<2, TERMS>(a, slot, row_block, pool, info.local, begin, count);
+    else if (count <= 96) tiles_mx_scaled_block<3, TERMS>(a, slot, row_block, pool, info.local, begin, count);
+    else tiles_mx_scaled_block<4, TERMS>(a, slot, row_block, pool, info.local, begin, count);
+}
+
+// One thread per (row, block of 32 columns): the E4M3 terms and their scales.
+__global__ void __launch_bounds__(256) fp8_split_kernel(const uint16_t* src, int half_in, int64_t items, int width, int terms,
+                                                        uint8_t* dst, uint8_t* scales) {
+    const int64_t item = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (item >= items) return;
+    const int blocks = width / kLaneColumns;
+    const int64_t row = item / blocks;
+    const int cb = static_cast<int>(item % blocks);
+    float x[32];
+    const uint16_t* from = src + row * width + cb * kLaneColumns;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const u32x4 raw = *(const MFQ_GLOBAL u32x4*)(from + 8 * j);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint16_t lo = static_cast<uint16_t>(raw[k] & 0xffffu), hi = static_cast<uint16_t>(raw[k] >> 16);
+            x[8 * j + 2 * k] = half_in ? half_bits_to_float(lo) : bf16_bits_to_float(lo);
+            x[8 * j + 2 * k + 1] = half_in ? half_bits_to_float(hi) : bf16_bits_to_float(hi);
+        }
+    }
+    for (int term = 0; term < terms; ++term) {
+        float largest = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) largest = fmaxf(largest, fabsf(x[i]));
+        const uint8_t s = block_scale_byte(largest);
+        const float down = scale_inverse(s), up = scale_value(s);
+        uint32_t words[8];
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            uint32_t word = 0u;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint8_t byte = e4m3_from_float(x[4 * w + k] * down);
+                x[4 * w + k] = x[4 * w + k] - e4m3_to_float(byte) * up;        // the residual: the next term's source
+                word |= static_cast<uint32_t>(byte) << (8 * k);
+            }
+            words[w] = word;
+        }
+        uint8_t* to = dst + (row * terms + term) * width + cb * kLaneColumns;
+        *reinterpret_cast<u32x4*>(to) = u32x4{words[0], words[1], words[2], words[3]};
+        *reinterpret_cast<u32x4*>(to + 16) = u32x4{words[4], words[5], words[6], words[7]};
+        scales[(row * terms + term) * blocks + cb] = s;
     }
 }
 
@@ -746,6 +917,30 @@ void launch_tiles_fast(const RowsArgs& args, int slots, int max_tiles, bool nvq,
     if (a.in_tiles != nullptr) hipLaunchKernelGGL(dev::moe_tiles_fast_kernel<true>, grid, dim3(256), bytes, stream, a);
     else hipLaunchKernelGGL(dev::moe_tiles_fast_kernel<false>, grid, dim3(256), bytes, stream, a);
     check_launch("moe_tiles_fast_kernel");
+}
+
+void launch_tiles_mx_scaled(const RowsArgs& args, int slots, int max_tiles, hipStream_t stream) {
+    if (max_tiles <= 0) return;
+    MFQ_REQUIRE(args.in_fp8 != nullptr && args.in_fp8_scales != nullptr && args.expert_info != nullptr &&
+                    (args.in_fp8_terms == 2 || args.in_fp8_terms == 3) && args.in_width % dev::kLaneColumns == 0,
+                "the block-scaled MFMA kernel needs the activations as two or three E4M3 terms");
+    RowsArgs a = args;
+    a.tile_slots = slots;
+    const int row_blocks = (args.out_rows + dev::kFastTileN - 1) / dev::kFastTileN;
+    const dim3 grid((max_tiles + 7) / 8 * 8 * row_blocks * slots);
+    if (a.in_fp8_terms == 2) hipLaunchKernelGGL(dev::moe_tiles_mx_scaled_kernel<2>, grid, dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(dev::moe_tiles_mx_scaled_kernel<3>, grid, dim3(256), 0, stream, a);
+    check_launch("moe_tiles_mx_scaled_kernel");
+}
+
+void launch_fp8_split(const void* src, int dtype, int rows, int width, int terms, uint8_t* dst, uint8_t* scales, hipStream_t stream) {
+    if (rows <= 0) return;
+    MFQ_REQUIRE(width % dev::kLaneColumns == 0 && dtype != MFQ_AMD_F32 && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
+                    (terms == 2 || terms == 3), "geometry is not served by the E4M3 split");
+    const int64_t items = static_cast<int64_t>(rows) * (width / dev::kLaneColumns);
+    hipLaunchKernelGGL(dev::fp8_split_kernel, dim3(static_cast<unsigned>((items + 255) / 256)), dim3(256), 0, stream,
+                       static_cast<const uint16_t*>(src), dtype == MFQ_AMD_F16 ? 1 : 0, items, width, terms, dst, scales);
+    check_launch("fp8_split_kernel");
 }
 
 void launch_tile_pack(const void* src, int dtype, int rows, int width, uint32_t layouts, uint16_t* dst, int64_t layout_stride,

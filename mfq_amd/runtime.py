@@ -218,7 +218,7 @@ class MfeFfnRuntime:
 
     def __init__(self, gate: MixedMoeRuntime, up: MixedMoeRuntime, down: MixedMoeRuntime, top_k: int,
                  max_tokens: int, x_dtype: torch.dtype = torch.bfloat16, out_dtype: torch.dtype = torch.float32,
-                 swiglu_limit: float = 0.0, decode_token_limit: int = 0, launch_mode: int = 0):
+                 swiglu_limit: float = 0.0, decode_token_limit: int = 0, launch_mode: int = 0, mx_scaled_mfma: bool = False):
         self._keep = (gate, up, down)
         self.top_k, self.max_tokens = top_k, max_tokens
         self.hidden = gate.neuron_len
@@ -231,6 +231,7 @@ class MfeFfnRuntime:
         config.swiglu_limit = swiglu_limit
         config.decode_token_limit = decode_token_limit
         config.launch_mode = launch_mode
+        config.mx_scaled_mfma = int(mx_scaled_mfma)
         handle = C.c_void_p()
         L.check(L.lib().mfq_amd_moe_ffn_create(C.byref(config), C.byref(handle)))
         self._handle = handle

@@ -111,3 +111,18 @@ def test_streaming_fetches_stay_inside_their_fields(tmp_path):
     done = subprocess.run([str(binary)], capture_output=True, text=True)
     assert done.returncode == 0, done.stderr
     assert "fetches inside their fields" in done.stdout and int(done.stdout.split()[0]) > 1_000_000
+
+
+def test_e4m3_split_rounding_and_scales(tmp_path):
+    """mfq_amd/csrc/fp8_split.h compiled for the host: E4M3 rounding against all byte values (nearest, ties to even,
+    saturation), the E8M0 block scale rule, and hi + lo adding up to bf16 sources."""
+    import shutil
+    import subprocess
+    compiler = shutil.which("g++") or shutil.which("hipcc")
+    if compiler is None:
+        pytest.skip("no host C++ compiler")
+    binary = tmp_path / "fp8_split_check"
+    subprocess.run([compiler, "-O2", "-std=c++17", str(ROOT / "tests" / "cpp" / "fp8_split_check.cpp"), "-o", str(binary)], check=True)
+    done = subprocess.run([str(binary)], capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
+    assert "roundings checked" in done.stdout

@@ -225,3 +225,38 @@ def test_token_counts_around_the_largest_decode_plan(tokens):
     err = rel_l2(out, oracle_layer(x, ids, weights, tensors))
     print(f"T={tokens} with decode limit 128, top-10: rel-L2 {err:.3e}")
     assert err <= TOL
+
+
+@pytest.mark.parametrize("case", ["uniform", "mixed", "f16", "ragged"])
+def test_prefill_mxfp4_on_the_block_scaled_mfma(case):
+    """mx_scaled_mfma = 1: prefill tiles of MXFP4 pools run on v_mfma_scale_f32_32x32x64_f8f6f4 with the weights as
+    stored (fp4 + E8M0 block scales) and the activations as E4M3 terms that add up to the source exactly (two for
+    bf16, three for fp16), the other formats on the fp16 tiles as before.  Same bar as every path: rel-L2 <= 1e-3."""
+    import torch
+    from mfq_amd import runtime as R
+    import synth
+    from test_gpu_moe import ALL_FORMATS, _layer
+    experts, hidden, inter, k, tokens, dtype = 6, 512, 128, 3, 150, torch.bfloat16
+    uniform, mix = None, ALL_FORMATS
+    if case == "uniform":
+        uniform = "MXFP4"
+    elif case == "mixed":
+        experts, k, tokens, mix = 24, 6, 300, (("MXFP4", 0.5), ("NINT4", 0.25), ("NVQ3J-L", 0.25))
+    elif case == "f16":
+        uniform, dtype = "MXFP4", torch.float16
+    else:
+        uniform, hidden, inter, tokens = "MXFP4", 96, 32, 70          # three and one lane blocks per row
+    tensors, runtimes, formats = _layer(f"test/mxscaled/{case}", experts, hidden, inter, "random", mix=mix, uniform=uniform)
+    assert any("MXFP4" in f for f in formats)
+    x = synth.normal(f"test/mxscaled/x/{case}", (tokens, hidden))
+    x = x.astype(np.float16).astype(np.float32) if dtype == torch.float16 else synth.to_bf16(x)
+    ids = synth.zipf_routes(f"test/mxscaled/ids/{case}", tokens, experts, k)
+    weights = np.full((tokens, k), 1.0 / k, dtype=np.float32)
+    args = (torch.from_numpy(x).to(dtype).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(weights).cuda())
+    expect = oracle_layer(x, ids, weights, tensors)
+    scaled = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens, x_dtype=dtype, mx_scaled_mfma=True).run(*args).cpu().numpy()
+    plain = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens, x_dtype=dtype).run(*args).cpu().numpy()
+    err_scaled, err_plain = rel_l2(scaled, expect), rel_l2(plain, expect)
+    print(f"MXFP4 prefill {case}: block-scaled MFMA {err_scaled:.3e}, fp16 tiles {err_plain:.3e}")
+    assert np.isfinite(scaled).all()
+    assert err_scaled <= TOL and err_plain <= TOL
