@@ -40,13 +40,17 @@ struct NoPrologue { __device__ __forceinline__ void operator()() const {} };
 // sequence is straight-line code, which lets the compiler wait for exactly the loads a slot needs;
 // SLOTS == 0: any number of rows, looped.  store(n, row, value) is called by one lane per (token, row).
 // IB: index bits of the NVQ format when known at compile time (0: looked up per row).
-template <int CLS, int LPR, int SLABS, int NT, int RING, int XMODE, int SLOTS, int IB = 0, class Store, class Prologue = NoPrologue>
+// LEVEL_WORDS (NINT classes, one lane block per lane): the group levels of a row slot come as level words (fetch_at.h)
+// that the wave shares, instead of two small loads per lane; the caller has checked nint_level_words_cover().
+template <int CLS, int LPR, int SLABS, int NT, int RING, int XMODE, int SLOTS, int IB = 0, bool LEVEL_WORDS = false, class Store,
+          class Prologue = NoPrologue>
 __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (&xs)[NT], int width, int row_begin,
                                           int row_end, int out_rows, Store&& store, Prologue&& prologue = Prologue()) {
     using C = FastClass<CLS>;
     constexpr int SUBS = kWave / LPR;          // rows per slot
     constexpr int R = RING < 4 ? RING : 4;     // slots whose totals are reduced together
     static_assert(RING % R == 0, "ring depth must be a multiple of the reduction width");
+    static_assert(!LEVEL_WORDS || (C::kNint && SLABS == 1), "level words serve NINT rows with one lane block per lane");
     const int lane = threadIdx.x % kWave;
     const int sub = lane / LPR, li = lane % LPR;
     const int slots = (row_end - row_begin + SUBS - 1) / SUBS;
@@ -55,11 +59,46 @@ __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (
 #pragma unroll
     for (int s = 0; s < SLABS; ++s) blocks[s] = lane_block<C::kGs>(li + LPR * s, width, c.groups);
 
+    // Level words.  As a loader, lanes 0..31 hold scale levels and lanes 32..63 minimum levels: word `word_j` of row
+    // `word_sub` of the slot; as a consumer, the lane takes the word that holds the levels of its block from lane
+    // `word_from` (+ 32 for the minima) and shifts them down by `word_shift`.
+    constexpr int kWordStride = nint_level_word_stride(C::kGs);
+    constexpr int kWordsPerRow = 32 / SUBS;
+    const uint8_t* word_array = nullptr;
+    int word_sub = 0, word_start = 0, word_from = 0, word_shift = 0;
+    if constexpr (LEVEL_WORDS) {
+        word_array = lane < 32 ? c.f1 : c.f2;
+        word_sub = (lane & 31) / kWordsPerRow;
+        word_start = nint_level_word_start(c.groups, kWordStride, (lane & 31) % kWordsPerRow);
+        const int first = C::kGs == 32 ? blocks[0].group : blocks[0].level_at;
+        const int word = nint_level_word_of(kWordStride, first);
+        word_from = 4 * (sub * kWordsPerRow + word);
+        word_shift = 8 * (first - nint_level_word_start(c.groups, kWordStride, word)) + (C::kGs == 32 ? 0 : blocks[0].level_shift);
+        blocks[0].level_shift = 0;
+    }
+
     auto fetch_slot = [&](int slot, FastRaw<CLS> (&raw)[SLABS]) {
         int row = row_begin + slot * SUBS + sub;
         row = row < out_rows ? row : out_rows - 1;
+        if constexpr (LEVEL_WORDS) {
+            raw[0] = fast_fetch<CLS, false>(c, blocks[0], row);
+            int from = row_begin + slot * SUBS + word_sub;
+            from = from < out_rows ? from : out_rows - 1;
+            raw[0].a = load_u32_unaligned(word_array + static_cast<uint32_t>(from) * static_cast<uint32_t>(c.groups) +
+                                          static_cast<uint32_t>(word_start));
+        } else {
 #pragma unroll
-        for (int s = 0; s < SLABS; ++s) raw[s] = fast_fetch<CLS>(c, blocks[s], row);
+            for (int s = 0; s < SLABS; ++s) raw[s] = fast_fetch<CLS>(c, blocks[s], row);
+        }
+    };
+    // The levels of the lane's block out of the slot's level words, in the form fast_accumulate() reads them.
+    auto with_levels = [&](const FastRaw<CLS>& raw) {
+        FastRaw<CLS> out = raw;
+        if constexpr (LEVEL_WORDS) {
+            out.a = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(word_from, static_cast<int>(raw.a))) >> word_shift;
+            out.b = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(word_from + 128, static_cast<int>(raw.a))) >> word_shift;
+        }
+        return out;
     };
 
     // Row scalars (NINT scale and minimum, NVQ anchor) of one pass over the ring: lane l holds those of
@@ -138,8 +177,8 @@ __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (
                 if (kScalars >= 2) rm = SUBS == 1 ? uniform_lane(scalars[1], k) : __shfl(scalars[1], k * SUBS + sub, kWave);
 #pragma unroll
                 for (int s = 0; s < SLABS; ++s) {
-                    if (s == 0 && !C::kNvq) fast_accumulate<CLS, NT, IB, false>(c, blocks[s], ring[d][s], rs, rm, x[s], row_v);
-                    else fast_accumulate<CLS, NT, IB>(c, blocks[s], ring[d][s], rs, rm, x[s], row_v);
+                    if (s == 0 && !C::kNvq) fast_accumulate<CLS, NT, IB, false>(c, blocks[s], with_levels(ring[d][s]), rs, rm, x[s], row_v);
+                    else fast_accumulate<CLS, NT, IB>(c, blocks[s], with_levels(ring[d][s]), rs, rm, x[s], row_v);
                 }
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
@@ -182,8 +221,8 @@ __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (
                 if (kScalars >= 2) rm = SUBS == 1 ? uniform_lane(scalars[1], d) : __shfl(scalars[1], d * SUBS + sub, kWave);
 #pragma unroll
                 for (int s = 0; s < SLABS; ++s) {
-                    if (s == 0 && !C::kNvq) fast_accumulate<CLS, NT, IB, false>(c, blocks[s], ring[d][s], rs, rm, x[s], row_v);
-                    else fast_accumulate<CLS, NT, IB>(c, blocks[s], ring[d][s], rs, rm, x[s], row_v);
+                    if (s == 0 && !C::kNvq) fast_accumulate<CLS, NT, IB, false>(c, blocks[s], with_levels(ring[d][s]), rs, rm, x[s], row_v);
+                    else fast_accumulate<CLS, NT, IB>(c, blocks[s], with_levels(ring[d][s]), rs, rm, x[s], row_v);
                 }
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {

@@ -53,6 +53,25 @@ MFQ_HD NintFetchAt nint_fetch_at(int row, int row_bytes, int groups, int bits, i
     return at;
 }
 
+// NINT level words (the row loop of the decode kernel): instead of every lane loading the two level bytes of its own
+// lane block, 32 / rows_per_slot lanes per row and level array load one dword each and the wave hands the bytes out
+// with lane permutes (one vector-memory instruction per row slot instead of two, each touching far fewer lanes).
+// Word j of a row starts at level stride * j, slid back so that it stays inside the row's own levels; stride 3 where a
+// lane block can begin at any level of a word (24- and 48-column groups), so that a block's two levels never straddle
+// two words, stride 4 where they cannot (16- and 32-column groups).
+MFQ_HD constexpr int nint_level_word_stride(int group_size) { return group_size == 16 || group_size == 32 ? 4 : 3; }
+// First level (index inside the row) of word j; needs groups >= 4.
+MFQ_HD int nint_level_word_start(int groups, int stride, int j) {
+    const int start = stride * j;
+    return start < groups - 4 ? start : groups - 4;
+}
+// The word that holds levels first and first + 1 (first <= groups - 2, or first <= groups - 1 when only one is wanted).
+MFQ_HD int nint_level_word_of(int stride, int first) { return first / stride; }
+// True when `words_per_row` words cover every lane block of a row.
+MFQ_HD bool nint_level_words_cover(int groups, int stride, int words_per_row) {
+    return groups >= 4 && nint_level_word_of(stride, groups - 1) < words_per_row;
+}
+
 // MXFP4: 16 bytes of nibbles at code_byte, one scale byte at scale_byte.
 struct MxFetchAt { uint32_t code_byte, scale_byte; };
 MFQ_HD MxFetchAt mx_fetch_at(int row, int row_bytes, const LaneBlock& b) {

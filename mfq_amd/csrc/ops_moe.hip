@@ -161,8 +161,15 @@ __device__ __forceinline__ void rows_fast_pair(const RowsArgs& a, const mfq_amd_
                             XMODE == kXScaled ? MFQ_AMD_F16 : a.in_dtype, XMODE == kXScaled ? true : a.in_vector_ok != 0,
                             hidden->scale}};
     constexpr int kRing = FastClass<CLS>::kRing < SLOTS || SLOTS == 0 ? FastClass<CLS>::kRing : SLOTS;
-    fast_rows<CLS, LPR, 1, 1, kRing, XMODE, SLOTS, IB>(ctx, xs, a.in_width, row_begin, row_end, a.out_rows,
-        [&](int, int row, float value) { out[row] = float_to_half_bits(value); }, prologue);
+    auto store = [&](int, int row, float value) { out[row] = float_to_half_bits(value); };
+    if constexpr (FastClass<CLS>::kNint && SLOTS > 0) {
+        // straight-line variants: the levels of a row slot as shared level words where the row's geometry allows
+        if (nint_level_words_cover(ctx.groups, nint_level_word_stride(FastClass<CLS>::kGs), 32 / (kWave / LPR))) {
+            fast_rows<CLS, LPR, 1, 1, kRing, XMODE, SLOTS, IB, true>(ctx, xs, a.in_width, row_begin, row_end, a.out_rows, store, prologue);
+            return;
+        }
+    }
+    fast_rows<CLS, LPR, 1, 1, kRing, XMODE, SLOTS, IB>(ctx, xs, a.in_width, row_begin, row_end, a.out_rows, store, prologue);
 }
 
 template <int CLS, int LPR, int XMODE, int SLOTS>

@@ -42,6 +42,30 @@ static void sweep_nint(int bits, int dwords, int width, int rows, int experts) {
                 require(static_cast<int64_t>(at.level_byte) + level_bytes <= static_cast<int64_t>(row + 1) * groups, "NINT levels leave their row", bits * 100 + GS, width, rows, experts, local, row, cb);
                 ++checked;
             }
+    // the level words of the decode row loop: each stays inside its row's levels, and every lane block finds both of
+    // its levels in the word it takes them from, below bit 32 after the shift
+    const int stride = nint_level_word_stride(GS);
+    for (int words_per_row : {32, 8}) {
+        const int lanes_per_row = words_per_row == 32 ? 64 : 16;
+        if (width > lanes_per_row * kLaneColumns || !nint_level_words_cover(groups, stride, words_per_row)) continue;
+        for (int row = 0; row < rows; ++row)
+            for (int j = 0; j < words_per_row; ++j) {
+                const int start = nint_level_word_start(groups, stride, j);
+                require(start >= 0 && start + 4 <= groups, "NINT level word leaves its row", bits * 100 + GS, width, rows, experts, 0, row, j);
+                ++checked;
+            }
+        for (int cb = 0; cb * kLaneColumns < width; ++cb) {
+            const LaneBlock b = lane_block<GS>(cb, width, groups);
+            const int first = GS == 32 ? b.group : b.level_at;
+            const int word = nint_level_word_of(stride, first);
+            const int start = nint_level_word_start(groups, stride, word);
+            const int shift = 8 * (first - start) + (GS == 32 ? 0 : b.level_shift);
+            require(word < words_per_row && first >= start && shift <= 24, "NINT level word does not hold the block's first level", bits * 100 + GS, width, rows, experts, 0, 0, cb);
+            // the second level is wanted only when the block spans two groups
+            if (b.sel != 0) require(shift <= 16, "NINT level word does not hold the block's second level", bits * 100 + GS, width, rows, experts, 0, 0, cb);
+            ++checked;
+        }
+    }
 }
 
 static void sweep_mx(int width, int rows, int experts) {
