@@ -202,7 +202,10 @@ typedef struct mfq_amd_moe_ffn_config {
                                   fp4 weights with their E8M0 scales as stored, activations as E4M3 terms that add up to the
                                   source exactly); 0: on the fp16 tiles like every other format.  Counterpart of
                                   mxfp4_moe_grouped_tensor_kernel (mfq/kernels/cuda/mx_matmul.cu:954). */
-    int32_t reserved[2];
+    int32_t expert_activation; /* 0: hidden = silu(gate) * up; 1: hidden = relu(up)^2 and no gate projection: gate.pool_count
+                                  must be 0 and swiglu_limit 0 (MfeFfnBatch::expert_activation, mfq/kernels/cuda/mfe_ffn.h:79-82,
+                                  :107-110) */
+    int32_t reserved[1];
 } mfq_amd_moe_ffn_config;
 
 /* create may allocate and synchronise; run allocates nothing, does not synchronise and can be
@@ -214,6 +217,19 @@ int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_amd_moe_ffn
 int32_t mfq_amd_moe_ffn_decode_limit(int32_t requested, int32_t top_k);
 int mfq_amd_moe_ffn_run(mfq_amd_moe_ffn* ffn, const void* x_dev, const int32_t* ids_dev,
                         const float* route_weights_dev, int32_t tokens, void* out_dev, void* stream);
+/* The layer's shared expert inside the FFN object (MfeFfnBatch::shared, shared_gate, shared_activation;
+ * mfq/kernels/cuda/mfe_ffn.h:45,60,79-82): a dense FFN (one expert per projection, gate NULL for shared_activation 1)
+ * that every token runs beside its routed experts.  set_shared may allocate and synchronise; the descriptors are
+ * copied, their device buffers stay borrowed.  run_shared is run() with the epilogue of mfe_ffn_down_reduce_kernel
+ * (mfq/kernels/cuda/mfe_ffn_device.cuh:1249-1263): out = half(sum_r w * pair) + shared_ffn(x)[half] * shared_gate[token]
+ * in fp32, written as config.out_dtype; shared_gate_dev holds one evaluated gate value per token (float32, float16 or
+ * bfloat16; with float16 the product is rounded to fp16 first, the reference's shared_product_half).  Allocates
+ * nothing, does not synchronise. */
+int mfq_amd_moe_ffn_set_shared(mfq_amd_moe_ffn* ffn, const mfq_amd_projection* gate, const mfq_amd_projection* up,
+                               const mfq_amd_projection* down, int32_t shared_activation);
+int mfq_amd_moe_ffn_run_shared(mfq_amd_moe_ffn* ffn, const void* x_dev, const int32_t* ids_dev, const float* route_weights_dev,
+                               const void* shared_gate_dev, int32_t shared_gate_dtype, int32_t tokens, void* out_dev,
+                               void* stream);
 /* The same layer with routing fused in: softmax top-k of logits_dev[tokens, experts] (arguments as
  * mfq_amd_topk) is selected inside the route-plan kernel when tokens <= min(decode_token_limit, 32),
  * by the top-k kernel otherwise.  Replaces the moe_topk_cuda + MfeFfnRuntime::run pair of calls

@@ -47,7 +47,8 @@ class MoeFfnConfig(C.Structure):
     _fields_ = [("gate", MoeTensor), ("up", MoeTensor), ("down", MoeTensor),
                 ("top_k", C.c_int32), ("max_tokens", C.c_int32), ("x_dtype", C.c_int32),
                 ("out_dtype", C.c_int32), ("swiglu_limit", C.c_float), ("decode_token_limit", C.c_int32),
-                ("launch_mode", C.c_int32), ("mx_scaled_mfma", C.c_int32), ("reserved", C.c_int32 * 2)]
+                ("launch_mode", C.c_int32), ("mx_scaled_mfma", C.c_int32), ("expert_activation", C.c_int32),
+                ("reserved", C.c_int32 * 1)]
 
 
 EXPORTS = {
@@ -80,6 +81,10 @@ EXPORTS = {
                                             C.c_int32, C.c_void_p, C.c_void_p]),
     "mfq_amd_moe_ffn_run_router": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_float, C.c_float,
                                             C.c_int32, C.c_void_p, C.c_void_p]),
+    "mfq_amd_moe_ffn_set_shared": (C.c_int, [C.c_void_p, C.POINTER(Projection), C.POINTER(Projection), C.POINTER(Projection),
+                                            C.c_int32]),
+    "mfq_amd_moe_ffn_run_shared": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
+                                            C.c_void_p, C.c_void_p]),
     "mfq_amd_moe_ffn_routes": (C.c_int, [C.c_void_p, c_void_pp, c_void_pp]),
     "mfq_amd_moe_ffn_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p,
                                       C.c_void_p]),

@@ -94,11 +94,19 @@ __device__ __forceinline__ float routing_expf(float x) {
     return input != input ? input : result;
 }
 
-// One SwiGLU output on fp16 bits.  limit > 0: clipped form in fp32.  Otherwise `table` maps the bits of a
+// `limit` value that selects the gate-less expert activation relu(up)^2 in swiglu_bits().
+constexpr float kActivationRelu2 = -1.0f;
+
+// One SwiGLU output on fp16 bits.  limit > 0: clipped form in fp32.  limit == 0: `table` maps the bits of a
 // half g to half(sigmoid(g)) and every product rounds to fp16, as the reference's fused path does
-// (mfq/kernels/cuda/moe.cu:1536-1542).
+// (mfq/kernels/cuda/moe.cu:1536-1542).  limit < 0 (kActivationRelu2): half(relu(up)^2), the gate is not read
+// (mfq/kernels/cuda/mfe_ffn.h:107-110, expert_activation == 1).
 __device__ __forceinline__ uint16_t swiglu_bits(uint16_t gb, uint16_t ub, float limit, const uint16_t* table) {
     const float g = half_bits_to_float(gb), u = half_bits_to_float(ub);
+    if (limit < 0.0f) {
+        const float positive = fmaxf(u, 0.0f);
+        return float_to_half_bits(positive * positive);
+    }
     if (limit > 0.0f) {
         const float clipped = fminf(g, limit);
         const float value = fminf(fmaxf(u, -limit), limit);

@@ -346,6 +346,33 @@ __global__ void shared_gate_kernel(const uint16_t* routed, const uint16_t* pairs
     out[index] = float_to_half_bits(value + term);
 }
 
+// Epilogue of a layer with a shared expert (the last lines of mfe_ffn_down_reduce_kernel,
+// mfq/kernels/cuda/mfe_ffn_device.cuh:1249-1263): routed = half(sum_r w * pair), routes ascending; contribution =
+// shared * gate in fp32 (rounded to fp16 when the gate values are fp16: shared_product_half); out = routed + contribution.
+// The gate values arrive evaluated (MfeFfnBatch::shared_gate), as float32, float16 or bfloat16.
+__global__ void shared_expert_reduce_kernel(const uint16_t* pairs, const float* weights, const int32_t* ids, int experts,
+                                            const uint16_t* shared, const void* gate, int gate_dtype, int tokens, int top_k, int width,
+                                            void* out, int out_dtype) {
+    const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index >= static_cast<int64_t>(tokens) * width) return;
+    const int64_t t = index / width, c = index % width;
+    float sum = 0.0f;
+    for (int r = 0; r < top_k; ++r) {
+        if (ids != nullptr && static_cast<unsigned>(ids[t * top_k + r]) >= static_cast<unsigned>(experts)) continue;
+        const float term = weights[t * top_k + r] * half_bits_to_float(pairs[(t * top_k + r) * width + c]);
+        sum = sum + term;
+    }
+    const float routed = half_bits_to_float(float_to_half_bits(sum));
+    const float g = gate_dtype == MFQ_AMD_F32 ? static_cast<const float*>(gate)[t]
+                  : gate_dtype == MFQ_AMD_F16 ? half_bits_to_float(static_cast<const uint16_t*>(gate)[t])
+                                              : bf16_bits_to_float(static_cast<const uint16_t*>(gate)[t]);
+    float contribution = half_bits_to_float(shared[index]) * g;
+    if (gate_dtype == MFQ_AMD_F16) contribution = half_bits_to_float(float_to_half_bits(contribution));
+    const float value = routed + contribution;
+    if (out_dtype == MFQ_AMD_F32) static_cast<float*>(out)[index] = value;
+    else static_cast<uint16_t*>(out)[index] = float_to_half_bits(value);
+}
+
 }  // namespace dev
 
 namespace {
@@ -601,6 +628,7 @@ struct mfq_amd_moe_ffn {
     uint16_t *d_gu = nullptr, *d_hidden = nullptr, *d_pairs = nullptr;
     const uint16_t* d_sigmoid = nullptr;   // the device's table: not owned
     int32_t* d_wave_base = nullptr;      // scratch of the two-kernel route plan
+    float activation_limit = 0.0f;       // what swiglu_bits() takes: the clamp of the gated activation, or kActivationRelu2
     float* d_logits = nullptr;           // router logits of run_router
     int32_t* d_route_ids = nullptr;      // routes selected by run_logits
     float* d_route_weights = nullptr;
@@ -613,6 +641,12 @@ struct mfq_amd_moe_ffn {
     hipStream_t last_stream = nullptr;
     const int32_t* last_ids = nullptr;   // routing of the last run (for touched_bytes)
     int last_pairs = 0;
+    // the layer's shared expert: a dense FFN of one expert that every token runs (set_shared), its route (expert 0, weight 1)
+    // and its output rows
+    mfq_amd_moe_ffn* shared = nullptr;
+    int32_t* d_shared_ids = nullptr;
+    float* d_shared_weights = nullptr;
+    uint16_t* d_shared_out = nullptr;
     bool decode_needs_items = true;   // some decode work runs on the exact kernels, which read the item lists
     bool timing = false;
     hipEvent_t events[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -620,8 +654,10 @@ struct mfq_amd_moe_ffn {
     ~mfq_amd_moe_ffn() {
         void* all[] = {d_pools, d_pool_class, d_pool_bytes, d_expert_pool, d_expert_info, d_expert_words, d_item_info, d_pair_items, d_items, d_class_offsets, d_tile_items,
                        d_tile_offsets, d_counts, d_bounds, d_tile_bounds, d_tile_experts, d_ids_dst, d_distinct,
-                       d_touched, d_gu, d_hidden, d_pairs, d_logits, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base, d_fp8, d_fp8_scales};
+                       d_touched, d_gu, d_hidden, d_pairs, d_logits, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base, d_fp8, d_fp8_scales,
+                       d_shared_ids, d_shared_weights, d_shared_out};
         for (void* p : all) if (p) (void)hipFree(p);
+        delete shared;
         for (hipEvent_t e : events) if (e) (void)hipEventDestroy(e);
     }
     void mark(int index, hipStream_t stream) {
@@ -640,15 +676,25 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
         MFQ_REQUIRE(c.out_dtype == MFQ_AMD_F32 || c.out_dtype == MFQ_AMD_F16, "output must be float32 or float16");
         MFQ_REQUIRE(c.launch_mode == 0 || c.launch_mode == 1, "unknown launch mode");
         MFQ_REQUIRE(c.mx_scaled_mfma == 0 || c.mx_scaled_mfma == 1, "mx_scaled_mfma must be 0 or 1");
-        MFQ_REQUIRE(c.gate.experts == c.up.experts && c.gate.experts == c.down.experts, "expert counts differ");
-        MFQ_REQUIRE(c.gate.neuron_len == c.up.neuron_len && c.gate.out_per_expert == c.up.out_per_expert &&
-                    c.down.neuron_len == c.gate.out_per_expert && c.down.out_per_expert == c.gate.neuron_len,
+        MFQ_REQUIRE(c.expert_activation == 0 || c.expert_activation == 1, "expert_activation must be 0 or 1");
+        MFQ_REQUIRE(c.swiglu_limit >= 0.0f, "swiglu_limit must not be negative");
+        const bool gated = c.expert_activation == 0;
+        if (gated) {
+            MFQ_REQUIRE(c.gate.experts == c.up.experts && c.gate.neuron_len == c.up.neuron_len &&
+                        c.gate.out_per_expert == c.up.out_per_expert, "gate and up shapes differ");
+        } else {
+            MFQ_REQUIRE(c.gate.pool_count == 0 && c.gate.pools == nullptr, "the relu-squared activation has no gate projection");
+            MFQ_REQUIRE(c.swiglu_limit == 0.0f, "swiglu_limit applies to the gated activation only");
+        }
+        MFQ_REQUIRE(c.up.experts == c.down.experts, "expert counts differ");
+        MFQ_REQUIRE(c.down.neuron_len == c.up.out_per_expert && c.down.out_per_expert == c.up.neuron_len,
                     "gate/up/down shapes do not form an FFN");
-        MFQ_REQUIRE(c.gate.experts <= kPlanMaxExperts, "at most 1024 experts");
-        f->experts = c.gate.experts; f->hidden = c.gate.neuron_len; f->intermediate = c.gate.out_per_expert;
+        MFQ_REQUIRE(c.up.experts <= kPlanMaxExperts, "at most 1024 experts");
+        f->experts = c.up.experts; f->hidden = c.up.neuron_len; f->intermediate = c.up.out_per_expert;
         f->top_k = c.top_k; f->max_tokens = c.max_tokens;
         f->decode_limit = mfq_amd_moe_ffn_decode_limit(c.decode_token_limit, c.top_k);
-        f->tables.add_slot(0, c.gate);
+        f->activation_limit = gated ? c.swiglu_limit : dev::kActivationRelu2;
+        if (gated) f->tables.add_slot(0, c.gate);      // no gate: the slot has no pools and every expert is absent from it
         f->tables.add_slot(1, c.up);
         f->tables.add_slot(2, c.down);
         // every expert must live in exactly one pool of every slot
@@ -675,7 +721,7 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
                 }
             }
             for (int e = 0; e < E; ++e)
-                if (owners[e] != 1) fail_unsupported("every expert must belong to exactly one pool of each projection");
+                if (owners[e] != (s == 0 && !gated ? 0 : 1)) fail_unsupported("every expert must belong to exactly one pool of each projection");
         }
         const size_t pools = f->tables.pools.size();
         f->d_pools = device_alloc<mfq_amd_projection>(pools);
@@ -767,7 +813,7 @@ namespace {
 // One layer.  `route`: select the routes from logits inside the plan kernel (decode sizes only) into
 // the object's own id and weight buffers; otherwise ids_dev / route_weights_dev are the caller's.
 void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, const float* route_weights_dev, int tokens,
-             void* out_dev, hipStream_t stream, const PlanRoute* route) {
+             void* out_dev, hipStream_t stream, const PlanRoute* route, bool reduce = true) {
     {
         f->last_stream = stream;
         f->last_ids = ids_dev;
@@ -906,18 +952,18 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         if (fuse_swiglu) {
             // no kernel of its own
         } else if (hidden_tiles) {
-            launch_swiglu_tiles(f->d_gu, f->d_gu + I, 2 * static_cast<int64_t>(I), I, pairs, f->config.swiglu_limit, f->d_sigmoid,
+            launch_swiglu_tiles(f->d_gu, f->d_gu + I, 2 * static_cast<int64_t>(I), I, pairs, f->activation_limit, f->d_sigmoid,
                                 ids_dev, f->d_expert_info + 2 * static_cast<int64_t>(E), E, f->d_hidden, stream);
         } else if (pack_hidden) {
             const size_t bytes = (static_cast<size_t>(I) * 2 + 15) / 16 * 16 + 64;
             hipLaunchKernelGGL(dev::swiglu_pack_kernel, dim3(pairs), dim3(256), bytes, stream, f->d_gu, f->d_gu + I,
-                               2 * static_cast<int64_t>(I), I, f->config.swiglu_limit, f->d_sigmoid, f->d_hidden,
+                               2 * static_cast<int64_t>(I), I, f->activation_limit, f->d_sigmoid, f->d_hidden,
                                f->d_hidden_packed, dev::xpack_row_dwords(I));
             check_launch("swiglu_pack_kernel");
         } else {
             const int64_t count = static_cast<int64_t>(pairs) * I;
             hipLaunchKernelGGL(dev::swiglu_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, stream,
-                               f->d_gu, f->d_gu + I, count, 2 * static_cast<int64_t>(I), static_cast<int64_t>(I), f->config.swiglu_limit,
+                               f->d_gu, f->d_gu + I, count, 2 * static_cast<int64_t>(I), static_cast<int64_t>(I), f->activation_limit,
                                f->d_sigmoid, f->d_hidden);
             check_launch("swiglu_kernel");
         }
@@ -929,12 +975,13 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         rows.out = f->d_pairs; rows.out_pair_stride = H; rows.out_slot_stride = 0;
         rows.slot_base = 2; rows.out_rows = H;
         rows.in_packed = pack_hidden ? f->d_hidden_packed : nullptr; rows.in_packed_stride = dev::xpack_row_dwords(I);
-        if (fuse_swiglu) { rows.gu = f->d_gu; rows.sigmoid = f->d_sigmoid; rows.swiglu_limit = f->config.swiglu_limit; }
+        if (fuse_swiglu) { rows.gu = f->d_gu; rows.sigmoid = f->d_sigmoid; rows.swiglu_limit = f->activation_limit; }
         rows.in_tiles = hidden_tiles ? f->d_hidden : nullptr; rows.in_tiles_layout_stride = 0;
         run_rows(2, 3);
         f->mark(4, stream);
 
-        launch_weighted_reduce(f->d_pairs, route_weights_dev, ids_dev, E, tokens, k, H, out_dev, f->config.out_dtype, stream);
+        // (a layer with a shared expert sums the pair rows in its own epilogue)
+        if (reduce) launch_weighted_reduce(f->d_pairs, route_weights_dev, ids_dev, E, tokens, k, H, out_dev, f->config.out_dtype, stream);
         f->mark(5, stream);
     }
 }
@@ -987,6 +1034,61 @@ extern "C" int mfq_amd_moe_ffn_run_router(mfq_amd_moe_ffn* f, const void* x_dev,
     });
     if (status != MFQ_AMD_OK || tokens == 0) return status;
     return mfq_amd_moe_ffn_run_logits(f, x_dev, f->d_logits, MFQ_AMD_F32, normalize, norm_floor, scale, tokens, out_dev, stream_ptr);
+}
+
+extern "C" int mfq_amd_moe_ffn_set_shared(mfq_amd_moe_ffn* f, const mfq_amd_projection* gate, const mfq_amd_projection* up,
+                                          const mfq_amd_projection* down, int32_t shared_activation) {
+    return guarded([&] {
+        MFQ_REQUIRE(f && up && down, "null argument");
+        MFQ_REQUIRE(shared_activation == 0 || shared_activation == 1, "shared_activation must be 0 or 1");
+        MFQ_REQUIRE((gate != nullptr) == (shared_activation == 0), "the gate projection is absent exactly for the relu-squared activation");
+        MFQ_REQUIRE(up->local_experts == 1 && down->local_experts == 1 && (!gate || gate->local_experts == 1),
+                    "the shared expert is a dense FFN: one expert per projection");
+        MFQ_REQUIRE(up->input_width == f->hidden && down->output_rows == f->hidden, "the shared expert does not fit the layer's width");
+        mfq_amd_moe_ffn_config c{};
+        auto dense = [](const mfq_amd_projection* p) {
+            mfq_amd_moe_tensor t{};
+            if (p != nullptr) { t.pools = p; t.pool_count = 1; t.experts = 1; t.out_per_expert = p->output_rows; t.neuron_len = p->input_width; }
+            return t;
+        };
+        c.gate = dense(gate); c.up = dense(up); c.down = dense(down);
+        c.top_k = 1; c.max_tokens = f->max_tokens; c.x_dtype = f->config.x_dtype; c.out_dtype = MFQ_AMD_F16;
+        c.swiglu_limit = shared_activation == 0 ? f->config.swiglu_limit : 0.0f;
+        c.decode_token_limit = f->config.decode_token_limit; c.launch_mode = f->config.launch_mode;
+        c.expert_activation = shared_activation;
+        mfq_amd_moe_ffn* made = nullptr;
+        if (mfq_amd_moe_ffn_create(&c, &made) != MFQ_AMD_OK) throw std::runtime_error(mfq_amd_last_error());
+        delete f->shared;
+        f->shared = made;
+        if (f->d_shared_ids == nullptr) {
+            f->d_shared_ids = device_alloc<int32_t>(f->max_tokens);
+            f->d_shared_weights = device_alloc<float>(f->max_tokens);
+            f->d_shared_out = device_alloc<uint16_t>(static_cast<size_t>(f->max_tokens) * f->hidden);
+            std::vector<float> ones(f->max_tokens, 1.0f);
+            MFQ_HIP(hipMemset(f->d_shared_ids, 0, sizeof(int32_t) * f->max_tokens));
+            MFQ_HIP(hipMemcpy(f->d_shared_weights, ones.data(), sizeof(float) * ones.size(), hipMemcpyHostToDevice));
+        }
+    });
+}
+
+extern "C" int mfq_amd_moe_ffn_run_shared(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, const float* route_weights_dev,
+                                          const void* shared_gate_dev, int32_t shared_gate_dtype, int32_t tokens, void* out_dev,
+                                          void* stream_ptr) {
+    return guarded([&] {
+        MFQ_REQUIRE(f && x_dev && ids_dev && route_weights_dev && shared_gate_dev && out_dev, "null argument");
+        MFQ_REQUIRE(f->shared != nullptr, "the layer has no shared expert: call mfq_amd_moe_ffn_set_shared first");
+        MFQ_REQUIRE(shared_gate_dtype >= MFQ_AMD_F32 && shared_gate_dtype <= MFQ_AMD_BF16, "shared gate values must be float32, float16 or bfloat16");
+        MFQ_REQUIRE(tokens >= 0 && tokens <= f->max_tokens, "token count exceeds the workspace capacity");
+        if (tokens == 0) return;
+        hipStream_t stream = as_stream(stream_ptr);
+        ffn_run(f, x_dev, ids_dev, route_weights_dev, tokens, nullptr, stream, nullptr, false);
+        ffn_run(f->shared, x_dev, f->d_shared_ids, f->d_shared_weights, tokens, f->d_shared_out, stream, nullptr);
+        const int64_t count = static_cast<int64_t>(tokens) * f->hidden;
+        hipLaunchKernelGGL(dev::shared_expert_reduce_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, stream,
+                           f->d_pairs, route_weights_dev, ids_dev, f->experts, f->d_shared_out, shared_gate_dev, shared_gate_dtype, tokens,
+                           f->top_k, f->hidden, out_dev, f->config.out_dtype);
+        check_launch("shared_expert_reduce_kernel");
+    });
 }
 
 extern "C" int mfq_amd_moe_ffn_routes(mfq_amd_moe_ffn* f, const int32_t** ids_dev, const float** weights_dev) {

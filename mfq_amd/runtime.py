@@ -216,16 +216,23 @@ class MixedMoeRuntime:
 class MfeFfnRuntime:
     """Routed expert FFN: gate/up -> SwiGLU -> down -> route-weighted reduce."""
 
-    def __init__(self, gate: MixedMoeRuntime, up: MixedMoeRuntime, down: MixedMoeRuntime, top_k: int,
+    def __init__(self, gate: MixedMoeRuntime | None, up: MixedMoeRuntime, down: MixedMoeRuntime, top_k: int,
                  max_tokens: int, x_dtype: torch.dtype = torch.bfloat16, out_dtype: torch.dtype = torch.float32,
-                 swiglu_limit: float = 0.0, decode_token_limit: int = 0, launch_mode: int = 0, mx_scaled_mfma: bool = False):
+                 swiglu_limit: float = 0.0, decode_token_limit: int = 0, launch_mode: int = 0, mx_scaled_mfma: bool = False,
+                 expert_activation: int = 0):
+        """expert_activation 1: hidden = relu(up)^2, ``gate`` must be None (a relu-squared bank has no gate descriptor)."""
+        if (gate is None) != (expert_activation == 1):
+            raise ValueError("the gate projection is absent exactly when expert_activation is 1")
         self._keep = (gate, up, down)
         self.top_k, self.max_tokens = top_k, max_tokens
-        self.hidden = gate.neuron_len
-        self.intermediate = gate.out_per_expert
+        self.hidden = up.neuron_len
+        self.intermediate = up.out_per_expert
         self.x_dtype, self.out_dtype = x_dtype, out_dtype
         config = L.MoeFfnConfig()
-        config.gate, config.up, config.down = gate.struct, up.struct, down.struct
+        if gate is not None:
+            config.gate = gate.struct
+        config.up, config.down = up.struct, down.struct
+        config.expert_activation = expert_activation
         config.top_k, config.max_tokens = top_k, max_tokens
         config.x_dtype, config.out_dtype = _DTYPES[x_dtype], _DTYPES[out_dtype]
         config.swiglu_limit = swiglu_limit
@@ -272,6 +279,30 @@ class MfeFfnRuntime:
             out = torch.empty((tokens, self.hidden), dtype=self.out_dtype, device="cuda")
         L.check(L.lib().mfq_amd_moe_ffn_run_router(self._handle, x.data_ptr(), router.data_ptr(), _dtype_code(router),
                                                    int(normalize), norm_floor, scale, tokens, out.data_ptr(), _stream()))
+        return out
+
+    def set_shared(self, gate: MixedMoeRuntime | None, up: MixedMoeRuntime, down: MixedMoeRuntime,
+                   shared_activation: int = 0) -> None:
+        """The layer's shared expert: dense one-expert projections (``MixedMoeRuntime.from_dense``); ``gate`` is None for
+        the relu-squared activation."""
+        self._shared_keep = (gate, up, down)
+        first = lambda runtime: C.byref(runtime.struct.pools[0]) if runtime is not None else None
+        L.check(L.lib().mfq_amd_moe_ffn_set_shared(self._handle, first(gate), first(up), first(down), shared_activation))
+
+    def run_shared(self, x: torch.Tensor, ids: torch.Tensor, route_weights: torch.Tensor, shared_gate: torch.Tensor,
+                   out: torch.Tensor | None = None) -> torch.Tensor:
+        """run() plus the shared expert: out = half(routed) + shared_ffn(x) * shared_gate[token]; ``shared_gate`` holds one
+        evaluated gate value per token (float32, float16 or bfloat16)."""
+        if x.dtype != self.x_dtype:
+            raise ValueError(f"x must be {self.x_dtype}")
+        x, ids, route_weights, shared_gate = x.contiguous(), ids.contiguous(), route_weights.contiguous(), shared_gate.contiguous()
+        tokens = x.shape[0]
+        if shared_gate.numel() != tokens:
+            raise ValueError("one shared gate value per token")
+        if out is None:
+            out = torch.empty((tokens, self.hidden), dtype=self.out_dtype, device="cuda")
+        L.check(L.lib().mfq_amd_moe_ffn_run_shared(self._handle, x.data_ptr(), ids.data_ptr(), route_weights.data_ptr(),
+                                                   shared_gate.data_ptr(), _dtype_code(shared_gate), tokens, out.data_ptr(), _stream()))
         return out
 
     def routes(self, tokens: int) -> tuple[torch.Tensor, torch.Tensor]:

@@ -471,6 +471,18 @@ uint16_t orc_swiglu_f16(uint16_t gate, uint16_t up, float swiglu_limit) {
     return orc_f32_to_f16(orc_f16_to_f32(first) * u);
 }
 
+/* Gate-less expert activation relu(up)^2 (mfq/kernels/cuda/mfe_ffn.h:107-110, expert_activation == 1): the square is
+ * taken in float and rounded to fp16 once. */
+uint16_t orc_relu2_f16(uint16_t up) {
+    float u = orc_f16_to_f32(up);
+    float positive = u > 0.0f ? u : 0.0f;
+    return orc_f32_to_f16(positive * positive);
+}
+
+void orc_relu2_array(const uint16_t* up, int64_t count, uint16_t* out) {
+    for (int64_t i = 0; i < count; ++i) out[i] = orc_relu2_f16(up[i]);
+}
+
 void orc_swiglu_array(const uint16_t* gate, const uint16_t* up, int64_t count, float swiglu_limit, uint16_t* out) {
     for (int64_t i = 0; i < count; ++i) out[i] = orc_swiglu_f16(gate[i], up[i], swiglu_limit);
 }

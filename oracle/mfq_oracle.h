@@ -131,6 +131,8 @@ void orc_projection_dequant(const orc_projection* p, float* out);
 /* ---- SwiGLU rounding chain (cuda/storage/moe_ffn_pipeline.cpp:154-169) ---- */
 uint16_t orc_swiglu_f16(uint16_t gate, uint16_t up, float swiglu_limit);
 void orc_swiglu_array(const uint16_t* gate, const uint16_t* up, int64_t count, float swiglu_limit, uint16_t* out);
+uint16_t orc_relu2_f16(uint16_t up);
+void orc_relu2_array(const uint16_t* up, int64_t count, uint16_t* out);
 /* x [count, width] f32 -> out [count, width] f32 through gate/up/down of one expert;
    gate/up/hidden scratch are [count, intermediate] */
 void orc_expert_ffn(const orc_projection* gate, const orc_projection* up, const orc_projection* down,

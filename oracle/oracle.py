@@ -78,6 +78,7 @@ def lib():
         L.orc_expf.restype = C.c_float; L.orc_expf.argtypes = [C.c_float]
         L.orc_swiglu_f16.restype = C.c_uint16; L.orc_swiglu_f16.argtypes = [C.c_uint16, C.c_uint16, C.c_float]
         L.orc_swiglu_array.argtypes = [_u16p, _u16p, C.c_int64, C.c_float, _u16p]
+        L.orc_relu2_array.argtypes = [_u16p, C.c_int64, _u16p]
         L.orc_nint_validate.restype = C.c_int; L.orc_nint_validate.argtypes = [C.POINTER(_NintView)]
         L.orc_projection_dequant.argtypes = [C.POINTER(_Projection), _f32p]
         L.orc_projection_rows.argtypes = [C.POINTER(_Projection), C.c_int, _f32p, C.c_int64, C.c_int64,
@@ -335,9 +336,21 @@ class Projection:
         return y
 
 
+def relu2_array(up_f16: np.ndarray) -> np.ndarray:
+    """half(relu(up)^2), the gate-less expert activation (mfq/kernels/cuda/mfe_ffn.h:107-110)."""
+    u = np.ascontiguousarray(up_f16, dtype=np.float16)
+    out = np.empty_like(u)
+    lib().orc_relu2_array(_ptr(u.view(np.uint16), _u16p), u.size, _ptr(out.view(np.uint16), _u16p))
+    return out
+
+
 def expert_ffn(gate: Projection, up: Projection, down: Projection, x: np.ndarray, order: int = 0,
-               swiglu_limit: float = 0.0) -> np.ndarray:
+               swiglu_limit: float = 0.0, activation: int = 0) -> np.ndarray:
+    """activation 1: hidden = half(relu(half(up . x))^2), no gate projection (``gate`` is ignored)."""
     x = np.ascontiguousarray(x, dtype=np.float32)
+    if activation == 1:
+        hidden = relu2_array(up.rows(x, order).astype(np.float16)).astype(np.float32)
+        return down.rows(hidden, order)
     count, inter = x.shape[0], gate.outputs
     g = np.empty((count, inter), dtype=np.float32)
     u = np.empty_like(g)
@@ -431,8 +444,22 @@ def weighted_reduce_shared_gate(pairs_f16: np.ndarray, weights: np.ndarray, shar
     return out
 
 
+def shared_expert_epilogue(routed_sum_f32: np.ndarray, shared_f16: np.ndarray, gate: np.ndarray) -> np.ndarray:
+    """The last lines of mfe_ffn_down_reduce_kernel (mfq/kernels/cuda/mfe_ffn_device.cuh:1249-1263): the route-ordered fp32
+    sum is rounded to fp16, the shared expert's fp16 output is multiplied with the token's evaluated gate value in fp32
+    (and the product rounded to fp16 when the gate values are fp16: shared_product_half), and the two are added in fp32.
+    ``gate``: [tokens] float32, float16 or bfloat16-as-float32 values."""
+    routed = np.asarray(routed_sum_f32, dtype=np.float32).astype(np.float16).astype(np.float32)
+    product_half = np.asarray(gate).dtype == np.float16
+    g = np.asarray(gate).astype(np.float32)[:, None]
+    contribution = np.asarray(shared_f16, dtype=np.float16).astype(np.float32) * g
+    if product_half:
+        contribution = contribution.astype(np.float16).astype(np.float32)
+    return (routed + contribution).astype(np.float32)
+
+
 def moe_layer(x: np.ndarray, ids: np.ndarray, weights: np.ndarray, expert_projections, order: int = 0,
-              swiglu_limit: float = 0.0) -> np.ndarray:
+              swiglu_limit: float = 0.0, activation: int = 0) -> np.ndarray:
     """Whole MoE FFN on the CPU: per routed pair the expert FFN of
     cuda/storage/moe_ffn_pipeline.cpp:142-180, pair outputs rounded to fp16
     (moe_ffn_pipeline.cpp:187 workspace type), then the route-ordered fp32 reduce.
@@ -448,7 +475,7 @@ def moe_layer(x: np.ndarray, ids: np.ndarray, weights: np.ndarray, expert_projec
     for e, slots in by_expert.items():
         gate, up, down = expert_projections(e)
         rows = np.stack([x[t] for t, _ in slots])
-        y = expert_ffn(gate, up, down, rows, order, swiglu_limit)
+        y = expert_ffn(gate, up, down, rows, order, swiglu_limit, activation)
         for (t, r), row in zip(slots, y):
             pairs[t, r] = row.astype(np.float16)
     return weighted_reduce(pairs, weights)

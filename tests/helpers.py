@@ -40,7 +40,9 @@ class OracleMoeTensor:
         return self._cache[expert]
 
 
-def oracle_layer(x_f32, ids, weights, tensors, order=0, swiglu_limit=0.0):
-    gate, up, down = (OracleMoeTensor(t) for t in tensors)
-    return O.moe_layer(x_f32, ids, weights, lambda e: (gate.projection(e), up.projection(e), down.projection(e)),
-                       order, swiglu_limit)
+def oracle_layer(x_f32, ids, weights, tensors, order=0, swiglu_limit=0.0, activation=0):
+    """tensors: (gate, up, down); gate may be None for the gate-less activation (activation=1)."""
+    gate, up, down = (OracleMoeTensor(t) if t is not None else None for t in tensors)
+    return O.moe_layer(x_f32, ids, weights,
+                       lambda e: (gate.projection(e) if gate is not None else None, up.projection(e), down.projection(e)),
+                       order, swiglu_limit, activation)

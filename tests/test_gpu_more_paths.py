@@ -96,6 +96,68 @@ def test_layer_with_clamped_swiglu_vs_oracle(tokens):
     assert rel_l2(free, expect) > 0.05, "the limit must change the result, or the test shows nothing"
 
 
+@pytest.mark.parametrize("tokens", [2, 16, 48])     # decode kernels (fused and separate activation) and the tile kernels
+def test_layer_with_relu_squared_experts_vs_oracle(tokens):
+    """expert_activation == 1 (mfq/kernels/cuda/mfe_ffn.h:79-82, :107-110): hidden = half(relu(up)^2), the bank has no
+    gate projection."""
+    import torch
+    from mfq_amd import runtime as R
+    from test_gpu_moe import _inputs, _layer
+    experts, hidden, inter, k = 24, 512, 128, 6
+    tensors, runtimes, _ = _layer("test/moe/random", experts, hidden, inter, "random")
+    x, ids, weights = _inputs(f"test/moe/relu2/in/{tokens}", tokens, experts, hidden, k)
+    args = (torch.from_numpy(x).to(torch.bfloat16).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(weights).cuda())
+    ffn = R.MfeFfnRuntime(None, runtimes[1], runtimes[2], top_k=k, max_tokens=64, expert_activation=1)
+    out = ffn.run(*args).cpu().numpy()
+    expect = oracle_layer(x, ids, weights, (None, tensors[1], tensors[2]), activation=1)
+    gated = oracle_layer(x, ids, weights, tensors)
+    err = rel_l2(out, expect)
+    print(f"relu^2 experts T={tokens}: rel-L2 {err:.3e}; distance to the gated layer {rel_l2(gated, expect):.3e}")
+    assert err <= TOL
+    assert rel_l2(gated, expect) > 0.5
+    with pytest.raises((ValueError, RuntimeError)):
+        R.MfeFfnRuntime(runtimes[0], runtimes[1], runtimes[2], top_k=k, max_tokens=64, expert_activation=1)
+
+
+@pytest.mark.parametrize("tokens,gate_dtype,activation", [(3, "f32", 0), (16, "f16", 0), (48, "bf16", 0), (5, "f32", 1)])
+def test_layer_with_shared_expert_inside_the_ffn(tokens, gate_dtype, activation):
+    """MfeFfnBatch::shared (mfq/kernels/cuda/mfe_ffn.h:45,60): routed experts and a dense shared expert in one call, the
+    epilogue of mfq/kernels/cuda/mfe_ffn_device.cuh:1249-1263.  Expectation: the oracle's routed sum and the oracle's
+    expert FFN of the shared projections, joined by two IEEE fp32 operations."""
+    import torch
+    from mfq_amd import runtime as R
+    import synth
+    from test_gpu_moe import _inputs, _layer
+    experts, hidden, inter, shared_inter, k = 24, 512, 128, 192, 6
+    tensors, runtimes, _ = _layer("test/moe/random", experts, hidden, inter, "random")
+    rng = np.random.default_rng(77)
+    dense = [synth.random_weights(fmt, rows, width, rng) for fmt, rows, width in
+             (("NINT4", shared_inter, hidden), ("NVQ3J-L", shared_inter, hidden), ("MXFP4", hidden, shared_inter))]
+    shared = [R.MixedMoeRuntime.from_dense(t) for t in dense]
+    x, ids, weights = _inputs(f"test/moe/shared/in/{tokens}", tokens, experts, hidden, k)
+    gate32 = rng.uniform(0.05, 0.95, tokens).astype(np.float32)
+    if gate_dtype == "f16":
+        gate_host, gate_dev = gate32.astype(np.float16), torch.from_numpy(gate32.astype(np.float16)).cuda()
+    elif gate_dtype == "bf16":
+        gate_host = synth.to_bf16(gate32)
+        gate_dev = torch.from_numpy(gate_host).to(torch.bfloat16).cuda()
+    else:
+        gate_host, gate_dev = gate32, torch.from_numpy(gate32).cuda()
+    ffn = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=64)
+    ffn.set_shared(None if activation else shared[0], shared[1], shared[2], activation)
+    out = ffn.run_shared(torch.from_numpy(x).to(torch.bfloat16).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(weights).cuda(),
+                         gate_dev).cpu().numpy()
+    routed = oracle_layer(x, ids, weights, tensors)
+    g, u, d = (O.Projection(O.runtime_layout(t)) for t in dense)
+    shared_out = O.expert_ffn(g, u, d, x, 0, 0.0, activation).astype(np.float16)
+    expect = O.shared_expert_epilogue(routed, shared_out, gate_host)
+    err = rel_l2(out, expect)
+    print(f"shared expert inside the FFN T={tokens} gate {gate_dtype} activation {activation}: rel-L2 {err:.3e}; "
+          f"share of the shared expert {rel_l2(routed, expect):.3e}")
+    assert err <= TOL
+    assert rel_l2(routed, expect) > 0.05
+
+
 @pytest.mark.parametrize("fmt", ["NINT4", "NVQ3J-L", "MXFP4", "NINT3-odd"])
 @pytest.mark.parametrize("tokens", [4, 40])
 def test_dense_single_expert_ffn_feeds_the_shared_gate_epilogue(fmt, tokens):

@@ -470,3 +470,21 @@ def test_reference_layer_driver_equals_expert_by_expert_rows():
     for pooled in (False, True):
         got = layer.run(pooled).copy()
         assert bits_equal(got, want), pooled
+
+
+def test_relu_squared_activation_against_exact_arithmetic():
+    """orc_relu2_f16 over every fp16 bit pattern.  The square of an fp16 value has at most 22 significant bits, so it
+    is exact in float32 and in float64 alike; rounding the float64 square to fp16 once is therefore the defined
+    result (mfq/kernels/cuda/mfe_ffn.h:107-110) reached by a different route."""
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    up = bits.view(np.float16)
+    got = O.relu2_array(up)
+    with np.errstate(over="ignore", invalid="ignore"):
+        wide = up.astype(np.float64)
+        expect = (np.where(wide > 0.0, wide, 0.0) ** 2).astype(np.float16)
+    finite = ~np.isnan(up)
+    assert np.array_equal(got.view(np.uint16)[finite], expect.view(np.uint16)[finite])
+    # negative inputs and both zeros give +0, overflow gives +inf, NaN gives 0 (fmaxf returns the other operand)
+    assert got[up < 0].view(np.uint16).max() == 0
+    assert np.isinf(got[up == np.float16(300.0)][0])
+    assert np.all(got[~finite].view(np.uint16) == 0)
