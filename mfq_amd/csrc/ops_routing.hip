@@ -152,35 +152,40 @@ __device__ __forceinline__ long long dpp64(long long v) {
 }
 __device__ __forceinline__ long long max64(long long a, long long b) { return a > b ? a : b; }
 
-// LDS scratch of one 32-lane group of topk_token.
+// LDS scratch of one lane group of topk_token.
 constexpr int kTopkCandidates = 64;
 struct TopkScratch {
     unsigned long long candidates[kTopkCandidates];   // (probability bits << 32) | ~expert: larger wins
-    int lane_best[32];                                // the best key of every lane
+    int lane_best[64];                                // the best key of every lane
     int selected[32];                                 // probability bits of rank r
     int threshold;                                    // top_k-th largest of lane_best
     int count;                                        // candidates found
 };
 
-// One 32-lane group per token, laid out like the reference kernels (lane owns experts lane,
-// lane+32, ...) so that the softmax denominator is summed in the same order
-// (mfq/kernels/cuda/moe.cu:1383-1446).  Selection works on integer keys: the bits of a non-negative
-// probability order like the value, an absent entry is -1, and ties go to the lower expert id.
+// One group of LANES lanes per token; lane l owns experts l, l + LANES, ... (SLOTS of them).  The softmax
+// denominator is summed in the order of the reference kernels, whose 32 lanes each add experts lane, lane + 32, ...
+// and then meet in a shuffle-down tree (mfq/kernels/cuda/moe.cu:1383-1446).  With LANES = 32 that is this layout;
+// with LANES = 64 (a whole wave per token: half the instructions per wave, and a wave issues one dependent
+// instruction every five cycles or so, which is what a small batch waits for) lane l < 32 fetches the numerators of
+// lane l + 32 and adds both sets alternately, which is the same sequence of additions.  Selection works on integer
+// keys: the bits of a non-negative probability order like the value, an absent entry is -1, and ties go to the lower
+// expert id; that order is total, so how the lanes share the entries does not change the result.
 //
-// The top_k-th largest of the 32 per-lane maxima is a lower bound of the top_k-th largest entry (at least top_k
+// The top_k-th largest of the per-lane maxima is a lower bound of the top_k-th largest entry (at least top_k
 // entries reach it), so only entries at or above it can be selected: usually one or two dozen.  They are
 // collected in LDS and every one counts the candidates that beat it; its rank is that count.  When more than
 // kTopkCandidates entries reach the bound (many equal probabilities, or the large ones crowded into few lanes) the
-// group falls back to one selection round per rank: the best of the 32 lane candidates by lane exchanges, and the
-// winning lane rescans its entries.  Both give the same ids: the order (probability, then lower id) is total.
+// group falls back to one selection round per rank: the best of the lane candidates by lane exchanges, and the
+// winning lane rescans its entries.  Both give the same ids.
 //
 // Every thread of the block calls it (block-wide barriers inside); groups with active == false select nothing.
 // `local_ids`, when given, also receives the ids (any address space, e.g. LDS).
-template <int SLOTS>
+template <int SLOTS, int LANES = 32>
 __device__ __forceinline__ void topk_token(const void* logits, int dtype, int token, bool active, int experts, int top_k,
                                            int normalize, float norm_floor, float scale, int32_t* ids,
                                            float* weights, int* local_ids, TopkScratch* scratch) {
-    const int lane = threadIdx.x & 31;
+    static_assert(LANES == 32 || LANES == 64, "a token takes half a wave or a whole one");
+    const int lane = threadIdx.x & (LANES - 1);
     const bool busy = __ballot(active) != 0ull;          // waves without a token only keep the barriers
     float cached[SLOTS];
     float total = 1.0f;
@@ -192,12 +197,12 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
         if (dtype == MFQ_AMD_F32) {
             const float* p = static_cast<const float*>(logits) + base;
 #pragma unroll
-            for (int slot = 0; slot < SLOTS; ++slot) cached[slot] = p[lane + slot * 32 < experts ? lane + slot * 32 : 0];
+            for (int slot = 0; slot < SLOTS; ++slot) cached[slot] = p[lane + slot * LANES < experts ? lane + slot * LANES : 0];
         } else {
             const uint16_t* p = static_cast<const uint16_t*>(logits) + base;
             uint16_t raw[SLOTS];
 #pragma unroll
-            for (int slot = 0; slot < SLOTS; ++slot) raw[slot] = p[lane + slot * 32 < experts ? lane + slot * 32 : 0];
+            for (int slot = 0; slot < SLOTS; ++slot) raw[slot] = p[lane + slot * LANES < experts ? lane + slot * LANES : 0];
 #pragma unroll
             for (int slot = 0; slot < SLOTS; ++slot)
                 cached[slot] = dtype == MFQ_AMD_F16 ? half_bits_to_float(raw[slot]) : bf16_bits_to_float(raw[slot]);
@@ -206,22 +211,38 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
 #pragma unroll
         for (int slot = 0; slot < SLOTS; ++slot) {
             const float v = cached[slot];
-            cached[slot] = lane + slot * 32 >= experts ? -__builtin_inff() : v != v ? -3.402823466e+38f : v;
+            cached[slot] = lane + slot * LANES >= experts ? -__builtin_inff() : v != v ? -3.402823466e+38f : v;
             maximum = fmaxf(maximum, cached[slot]);
         }
 #pragma unroll
-        for (int offset = 16; offset > 0; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset, 32));
+        for (int offset = LANES / 2; offset > 0; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset, LANES));
         float sum = 0.0f;
+        if constexpr (LANES == 32) {
 #pragma unroll
-        for (int slot = 0; slot < SLOTS; ++slot) {
-            if (lane + slot * 32 < experts) {
-                cached[slot] = routing_expf(cached[slot] - maximum);
-                sum = sum + cached[slot];
-            } else {
-                cached[slot] = -1.0f;                     // absent: the bits of a negative number are a negative key
+            for (int slot = 0; slot < SLOTS; ++slot) {
+                if (lane + slot * 32 < experts) {
+                    cached[slot] = routing_expf(cached[slot] - maximum);
+                    sum = sum + cached[slot];
+                } else {
+                    cached[slot] = -1.0f;                     // absent: the bits of a negative number are a negative key
+                }
+            }
+        } else {
+#pragma unroll
+            for (int slot = 0; slot < SLOTS; ++slot)
+                cached[slot] = lane + slot * 64 < experts ? routing_expf(cached[slot] - maximum) : -1.0f;
+            // lane l < 32 adds experts l, l + 32, l + 64, ... in that order: its own entries and those of lane l + 32 in turn
+            // (the upper lanes run the same code on values nobody reads)
+#pragma unroll
+            for (int slot = 0; slot < SLOTS; ++slot) {
+                const float other = __shfl_xor(cached[slot], 32, 64);
+                const int first = (lane & 31) + slot * 64;
+                if (first < experts) sum = sum + cached[slot];
+                if (first + 32 < experts) sum = sum + other;
             }
         }
         total = tree32_sum(sum);
+        if constexpr (LANES == 64) total = __shfl(total, 0, 64);
         // The numerators order like the probabilities (division by the common total is monotone), except that
         // numerators a few units in the last place apart may give the same probability: the bound below is taken
         // on the numerators and lowered by that much, the probabilities themselves are computed for candidates only.
@@ -238,7 +259,7 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
         // the top_k-th largest lane maximum: the smallest one that fewer than top_k others exceed
         int greater = 0;
 #pragma unroll
-        for (int i = 0; i < 32; i += 4) {
+        for (int i = 0; i < LANES; i += 4) {
             const int4 v = *reinterpret_cast<const int4*>(&scratch->lane_best[i]);
             greater += (v.x > lane_best) + (v.y > lane_best) + (v.z > lane_best) + (v.w > lane_best);
         }
@@ -256,7 +277,7 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
             const uint32_t bits = __float_as_uint(cached[slot]);
             if (active && static_cast<int>(bits) >= bound) {
                 if (at < kTopkCandidates)
-                    scratch->candidates[at] = (static_cast<unsigned long long>(bits) << 32) | static_cast<uint32_t>(~(lane + 32 * slot));
+                    scratch->candidates[at] = (static_cast<unsigned long long>(bits) << 32) | static_cast<uint32_t>(~(lane + LANES * slot));
                 ++at;
             }
         }
@@ -265,12 +286,12 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
     const int found = busy ? scratch->count : 0;
     // (numerators below 2^-100 can give subnormal probabilities, where many more numerators share one quotient)
     const bool by_rounds = active && (found > kTopkCandidates || found < top_k || scratch->threshold < 0x0D800000);
-    unsigned long long mine2[kTopkCandidates / 32];
+    unsigned long long mine2[kTopkCandidates / LANES];
     if (busy && active && !by_rounds) {
         // numerator -> probability, for the candidates only
 #pragma unroll
-        for (int j = 0; j < kTopkCandidates / 32; ++j) {
-            const int at = lane + 32 * j;
+        for (int j = 0; j < kTopkCandidates / LANES; ++j) {
+            const int at = lane + LANES * j;
             mine2[j] = 0ull;
             if (at < found) {
                 const unsigned long long c = scratch->candidates[at];
@@ -282,14 +303,14 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
     __syncthreads();
     if (busy && active && !by_rounds) {
 #pragma unroll
-        for (int j = 0; j < kTopkCandidates / 32; ++j)
-            if (lane + 32 * j < found) scratch->candidates[lane + 32 * j] = mine2[j];
+        for (int j = 0; j < kTopkCandidates / LANES; ++j)
+            if (lane + LANES * j < found) scratch->candidates[lane + LANES * j] = mine2[j];
     }
     __syncthreads();
     if (busy && active && !by_rounds) {
 #pragma unroll
-        for (int j = 0; j < kTopkCandidates / 32; ++j) {
-            if (lane + 32 * j >= found) continue;
+        for (int j = 0; j < kTopkCandidates / LANES; ++j) {
+            if (lane + LANES * j >= found) continue;
             const unsigned long long me = mine2[j];
             int rank = 0;
             for (int i = 0; i < found; ++i) rank += scratch->candidates[i] > me;
@@ -306,7 +327,7 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
         int key[SLOTS];
 #pragma unroll
         for (int slot = 0; slot < SLOTS; ++slot)
-            key[slot] = lane + slot * 32 < experts ? static_cast<int>(__float_as_uint(cached[slot] / total)) : -1;
+            key[slot] = lane + slot * LANES < experts ? static_cast<int>(__float_as_uint(cached[slot] / total)) : -1;
         auto local_best = [&](int& best, int& best_slot) {
             best = -1; best_slot = 0;
 #pragma unroll
@@ -317,12 +338,13 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
         local_best(best, best_slot);
         for (int rank = 0; rank < top_k; ++rank) {
             // candidate of this lane: (probability bits, ~expert); larger wins
-            long long candidate = (static_cast<long long>(best) << 32) | static_cast<uint32_t>(~(lane + 32 * best_slot));
+            long long candidate = (static_cast<long long>(best) << 32) | static_cast<uint32_t>(~(lane + LANES * best_slot));
             candidate = max64(candidate, dpp64<0xB1>(candidate));    // lane ^ 1
             candidate = max64(candidate, dpp64<0x4E>(candidate));    // lane ^ 2
             candidate = max64(candidate, dpp64<0x141>(candidate));   // mirror inside 8 lanes
             candidate = max64(candidate, dpp64<0x140>(candidate));   // mirror inside 16 lanes
-            candidate = max64(candidate, __shfl_xor(candidate, 16, 32));
+            candidate = max64(candidate, __shfl_xor(candidate, 16, LANES));
+            if constexpr (LANES == 64) candidate = max64(candidate, __shfl_xor(candidate, 32, 64));
             const int expert = static_cast<int>(~static_cast<uint32_t>(candidate));
             const int bits = static_cast<int>(candidate >> 32);
             if (lane == rank) {
@@ -330,8 +352,8 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
                 ids[static_cast<int64_t>(token) * top_k + rank] = expert;
                 if (local_ids != nullptr) local_ids[token * top_k + rank] = expert;
             }
-            if (lane == (expert & 31)) {
-                const int taken = expert >> 5;
+            if (lane == (expert & (LANES - 1))) {
+                const int taken = expert / LANES;
 #pragma unroll
                 for (int slot = 0; slot < SLOTS; ++slot)
                     if (slot == taken) key[slot] = -1;
@@ -686,10 +708,18 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_small_kernel(PlanArgs
     if (TOPK_SLOTS > 0) {
         expert_of[tid] = -1;
         __syncthreads();
-        const int token = tid >> 5;
-        topk_token<(TOPK_SLOTS > 0 ? TOPK_SLOTS : 1)>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
-                                                      a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
-                                                      a.route.weights_out, expert_of, &topk_scratch[token]);
+        // a whole wave per token while the block has waves to spare, half a wave beyond that
+        if (a.route.tokens <= kPlanThreads / 128) {
+            const int token = tid >> 6;
+            topk_token<(TOPK_SLOTS >= 2 ? TOPK_SLOTS / 2 : 1), 64>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
+                                                                   a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
+                                                                   a.route.weights_out, expert_of, &topk_scratch[token]);
+        } else {
+            const int token = tid >> 5;
+            topk_token<(TOPK_SLOTS > 0 ? TOPK_SLOTS : 1)>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
+                                                          a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
+                                                          a.route.weights_out, expert_of, &topk_scratch[token]);
+        }
         __syncthreads();
         expert = expert_of[tid];
     } else {
@@ -935,10 +965,18 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_pairs_kernel(PlanArgs
 #pragma unroll
     for (int s = 0; s < kSlots; ++s) words[s] = s < x.slots && tid < E ? x.expert_words[s * E + tid] : kExpertAbsent;
     if (TOPK_SLOTS > 0) {
-        const int token = tid >> 5;
-        topk_token<(TOPK_SLOTS > 0 ? TOPK_SLOTS : 1)>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
-                                                      a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
-                                                      a.route.weights_out, expert_of, &topk_scratch[token]);
+        // a whole wave per token while the block has waves to spare, half a wave beyond that
+        if (a.route.tokens <= kPlanThreads / 128) {
+            const int token = tid >> 6;
+            topk_token<(TOPK_SLOTS >= 2 ? TOPK_SLOTS / 2 : 1), 64>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
+                                                                   a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
+                                                                   a.route.weights_out, expert_of, &topk_scratch[token]);
+        } else {
+            const int token = tid >> 5;
+            topk_token<(TOPK_SLOTS > 0 ? TOPK_SLOTS : 1)>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
+                                                          a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
+                                                          a.route.weights_out, expert_of, &topk_scratch[token]);
+        }
     } else if (tid < P) {
         expert_of[tid] = a.ids[tid];
     }
