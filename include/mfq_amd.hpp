@@ -115,6 +115,8 @@ struct MfeFfnOptions {
     float swiglu_limit = 0.0f;
     int decode_token_limit = 0;   /* 0 = the library's default */
     int launch_mode = 0;
+    int expert_activation = 0;    /* 1: relu(up)^2, the gate projection is then a null pointer */
+    bool mx_scaled_mfma = false;  /* prefill tiles of MXFP4 pools on the block-scaled MFMA (an experiment) */
 };
 
 /* The routed FFN of one layer: gate and up per routed pair, SwiGLU, down per pair, route-weighted reduce. */
@@ -123,10 +125,11 @@ public:
     /* projections = {gate, up, down}; they must outlive this object (their device buffers are borrowed). */
     MfeFfnRuntime(const std::array<const MixedMoeRuntime*, 3>& projections, const MfeFfnOptions& options)
         : top_k_(options.top_k), max_tokens_(options.max_tokens) {
-        for (const MixedMoeRuntime* p : projections)
-            if (!p) throw Error(MFQ_AMD_ERR_INVALID, "MfeFfnRuntime needs gate, up and down projections");
+        const bool gated = options.expert_activation == 0;
+        if (!projections[1] || !projections[2] || (projections[0] != nullptr) != gated)
+            throw Error(MFQ_AMD_ERR_INVALID, "MfeFfnRuntime needs up and down projections, and gate exactly for the gated activation");
         mfq_amd_moe_ffn_config config{};
-        config.gate = projections[0]->tensor();
+        if (gated) config.gate = projections[0]->tensor();
         config.up = projections[1]->tensor();
         config.down = projections[2]->tensor();
         config.top_k = options.top_k;
@@ -136,6 +139,8 @@ public:
         config.swiglu_limit = options.swiglu_limit;
         config.decode_token_limit = options.decode_token_limit;
         config.launch_mode = options.launch_mode;
+        config.expert_activation = options.expert_activation;
+        config.mx_scaled_mfma = options.mx_scaled_mfma ? 1 : 0;
         check(mfq_amd_moe_ffn_create(&config, &ffn_));
     }
     MfeFfnRuntime(const MfeFfnRuntime&) = delete;
@@ -156,6 +161,23 @@ public:
                     bool normalize = true, float norm_floor = 1e-20f, float scale = 1.0f) {
         check(mfq_amd_moe_ffn_run_logits(ffn_, x, logits, logits_dtype, normalize ? 1 : 0, norm_floor, scale, tokens, out,
                                          stream));
+    }
+    /* The same from x and the router weights[experts, hidden]: the router matmul runs in front. */
+    void run_router(const void* x, const void* router, int router_dtype, int tokens, void* out, void* stream,
+                    bool normalize = true, float norm_floor = 1e-20f, float scale = 1.0f) {
+        check(mfq_amd_moe_ffn_run_router(ffn_, x, router, router_dtype, normalize ? 1 : 0, norm_floor, scale, tokens, out, stream));
+    }
+    /* The layer's shared expert (MfeFfnBatch::shared): dense projections with one expert each; gate is null for
+     * shared_activation 1.  The descriptors are copied, their device buffers stay borrowed. */
+    void set_shared(const mfq_amd_projection* gate, const mfq_amd_projection* up, const mfq_amd_projection* down,
+                    int shared_activation = 0) {
+        check(mfq_amd_moe_ffn_set_shared(ffn_, gate, up, down, shared_activation));
+    }
+    /* run() plus the shared expert: out = half(routed) + shared_ffn(x) * shared_gate[token] (one evaluated gate value per
+     * token, of shared_gate_dtype). */
+    void run_shared(const void* x, const std::int32_t* ids, const float* route_weights, const void* shared_gate,
+                    int shared_gate_dtype, int tokens, void* out, void* stream) {
+        check(mfq_amd_moe_ffn_run_shared(ffn_, x, ids, route_weights, shared_gate, shared_gate_dtype, tokens, out, stream));
     }
     /* Device pointers to the routes run_logits selected: ids i32 [tokens, k], weights f32 [tokens, k]. */
     std::pair<const std::int32_t*, const float*> routes() {
