@@ -990,9 +990,10 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
 extern "C" int mfq_amd_moe_ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev,
                                    const float* route_weights_dev, int32_t tokens, void* out_dev, void* stream_ptr) {
     return guarded([&] {
-        MFQ_REQUIRE(f && x_dev && ids_dev && route_weights_dev && out_dev, "null argument");
+        MFQ_REQUIRE(f, "null argument");
         MFQ_REQUIRE(tokens >= 0 && tokens <= f->max_tokens, "token count exceeds the workspace capacity");
-        if (tokens == 0) return;
+        if (tokens == 0) return;                   // an empty batch: nothing is read, the buffers may be null
+        MFQ_REQUIRE(x_dev && ids_dev && route_weights_dev && out_dev, "null argument");
         ffn_run(f, x_dev, ids_dev, route_weights_dev, tokens, out_dev, as_stream(stream_ptr), nullptr);
     });
 }
@@ -1001,11 +1002,12 @@ extern "C" int mfq_amd_moe_ffn_run_logits(mfq_amd_moe_ffn* f, const void* x_dev,
                                           int32_t logits_dtype, int32_t normalize, float norm_floor, float scale,
                                           int32_t tokens, void* out_dev, void* stream_ptr) {
     return guarded([&] {
-        MFQ_REQUIRE(f && x_dev && logits_dev && out_dev, "null argument");
+        MFQ_REQUIRE(f, "null argument");
         MFQ_REQUIRE(tokens >= 0 && tokens <= f->max_tokens, "token count exceeds the workspace capacity");
         MFQ_REQUIRE(logits_dtype >= MFQ_AMD_F32 && logits_dtype <= MFQ_AMD_BF16, "logits must be float32, float16 or bfloat16");
         MFQ_REQUIRE(f->top_k <= f->experts, "top_k exceeds the number of experts");
         if (tokens == 0) return;
+        MFQ_REQUIRE(x_dev && logits_dev && out_dev, "null argument");
         hipStream_t stream = as_stream(stream_ptr);
         PlanRoute route{};
         route.logits = logits_dev; route.dtype = logits_dtype; route.tokens = tokens; route.normalize = normalize;
@@ -1025,10 +1027,11 @@ extern "C" int mfq_amd_moe_ffn_run_router(mfq_amd_moe_ffn* f, const void* x_dev,
                                           int32_t normalize, float norm_floor, float scale, int32_t tokens, void* out_dev,
                                           void* stream_ptr) {
     const int status = guarded([&] {
-        MFQ_REQUIRE(f && x_dev && router_dev && out_dev, "null argument");
+        MFQ_REQUIRE(f, "null argument");
         MFQ_REQUIRE(tokens >= 0 && tokens <= f->max_tokens, "token count exceeds the workspace capacity");
         MFQ_REQUIRE(router_dtype >= MFQ_AMD_F32 && router_dtype <= MFQ_AMD_BF16, "router weights must be float32, float16 or bfloat16");
         if (tokens == 0) return;
+        MFQ_REQUIRE(x_dev && router_dev && out_dev, "null argument");
         launch_router_logits(x_dev, f->config.x_dtype, router_dev, router_dtype, tokens, f->experts, f->hidden, f->d_logits,
                              as_stream(stream_ptr));
     });
@@ -1075,11 +1078,12 @@ extern "C" int mfq_amd_moe_ffn_run_shared(mfq_amd_moe_ffn* f, const void* x_dev,
                                           const void* shared_gate_dev, int32_t shared_gate_dtype, int32_t tokens, void* out_dev,
                                           void* stream_ptr) {
     return guarded([&] {
-        MFQ_REQUIRE(f && x_dev && ids_dev && route_weights_dev && shared_gate_dev && out_dev, "null argument");
+        MFQ_REQUIRE(f, "null argument");
         MFQ_REQUIRE(f->shared != nullptr, "the layer has no shared expert: call mfq_amd_moe_ffn_set_shared first");
         MFQ_REQUIRE(shared_gate_dtype >= MFQ_AMD_F32 && shared_gate_dtype <= MFQ_AMD_BF16, "shared gate values must be float32, float16 or bfloat16");
         MFQ_REQUIRE(tokens >= 0 && tokens <= f->max_tokens, "token count exceeds the workspace capacity");
         if (tokens == 0) return;
+        MFQ_REQUIRE(x_dev && ids_dev && route_weights_dev && shared_gate_dev && out_dev, "null argument");
         hipStream_t stream = as_stream(stream_ptr);
         ffn_run(f, x_dev, ids_dev, route_weights_dev, tokens, nullptr, stream, nullptr, false);
         ffn_run(f->shared, x_dev, f->d_shared_ids, f->d_shared_weights, tokens, f->d_shared_out, stream, nullptr);

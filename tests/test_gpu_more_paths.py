@@ -158,6 +158,45 @@ def test_layer_with_shared_expert_inside_the_ffn(tokens, gate_dtype, activation)
     assert rel_l2(routed, expect) > 0.05
 
 
+@pytest.mark.parametrize("tokens", [5, 16, 40])      # small and sorted decode plans, prefill tiles
+def test_layer_with_absent_and_repeated_routes(tokens):
+    """Routes whose expert id lies outside [0, experts) add nothing (cuda/ops/moe.cpp:257-320 skips them in the plan),
+    and a token may name one expert twice (two pairs of one expert and token).  Also: an empty batch is a no-op, and a
+    batch of exactly max_tokens runs."""
+    import torch
+    from mfq_amd import runtime as R
+    from test_gpu_moe import _inputs, _layer
+    experts, hidden, inter, k = 24, 512, 128, 6
+    tensors, runtimes, _ = _layer("test/moe/random", experts, hidden, inter, "random")
+    x, ids, weights = _inputs(f"test/moe/edge/in/{tokens}", tokens, experts, hidden, k)
+    ids = ids.copy()
+    rng = np.random.default_rng(tokens)
+    absent = rng.random(ids.shape) < 0.2
+    ids[absent] = np.where(rng.random(int(absent.sum())) < 0.5, -1, experts + 3)
+    repeated = (rng.random(tokens) < 0.5) & ~absent[:, 0] & ~absent[:, 1]
+    ids[repeated, 1] = ids[repeated, 0]
+    assert absent.any() and repeated.any()
+    ffn = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens)          # the batch fills the workspace exactly
+    xd = torch.from_numpy(x).to(torch.bfloat16).cuda()
+    out = ffn.run(xd, torch.from_numpy(ids).cuda(), torch.from_numpy(weights).cuda()).cpu().numpy()
+    # the oracle sees the absent routes as routes of expert 0 with weight zero
+    seen_ids, seen_weights = np.where(absent, 0, ids).astype(np.int32), np.where(absent, 0.0, weights).astype(np.float32)
+    expect = oracle_layer(x, seen_ids, seen_weights, tensors)
+    err = rel_l2(out, expect)
+    print(f"absent and repeated routes T={tokens}: rel-L2 {err:.3e} ({int(absent.sum())} absent, {int(repeated.sum())} repeated)")
+    assert err <= TOL
+    # a token whose routes are all absent gets zeros
+    none = np.full_like(ids, -1)
+    zeros = ffn.run(xd, torch.from_numpy(none).cuda(), torch.from_numpy(weights).cuda()).cpu().numpy()
+    assert not zeros.any()
+    # an empty batch leaves the output untouched and reports success
+    marker = torch.full((1, hidden), 7.0, dtype=torch.float32, device="cuda")
+    ffn.run(xd[:0], torch.from_numpy(ids[:0]).cuda(), torch.from_numpy(weights[:0]).cuda(), marker[:0])
+    assert float(marker.min()) == 7.0
+    with pytest.raises((ValueError, RuntimeError)):
+        R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens - 1).run(xd, torch.from_numpy(ids).cuda(), torch.from_numpy(weights).cuda())
+
+
 @pytest.mark.parametrize("fmt", ["NINT4", "NVQ3J-L", "MXFP4", "NINT3-odd"])
 @pytest.mark.parametrize("tokens", [4, 40])
 def test_dense_single_expert_ffn_feeds_the_shared_gate_epilogue(fmt, tokens):
