@@ -889,11 +889,15 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         };
         const int active_bound = pairs < E ? pairs : E;
         int rows_in_width = 0;
-        // enough blocks to fill the chip at small batches, long row runs per wave at large ones
+        // Enough blocks to fill the chip at small batches, long row runs per wave at large ones: the tallest block with
+        // straight-line code (16 row slots per wave for wide rows, 8 for rows of at most 512 columns), halved while the
+        // launch has fewer blocks than the chip holds at once (measured at 512 experts x (2048 <-> 512), top-10: a floor
+        // of 1024 blocks against 2048 gives 41.9 vs 43.1 us per step at batch 4 and 57.2 vs 60.1 us at batch 8, and
+        // leaves batches 1, 2 and 16 where they were; 512 is slower everywhere)
         auto rows_per_block = [&](int out_rows, int slots) {
-            int rows = 256;
             const int least = rows_fast_min_block(rows_in_width);
-            while (rows > least && static_cast<int64_t>(pairs) * slots * ((out_rows + rows - 1) / rows) < 2048) rows /= 2;
+            int rows = rows_in_width <= 16 * dev::kLaneColumns ? 128 : 64;
+            while (rows > least && static_cast<int64_t>(pairs) * slots * ((out_rows + rows - 1) / rows) < 1024) rows /= 2;
             return rows;
         };
         auto run_rows = [&](int slot_lo, int slot_hi) {
