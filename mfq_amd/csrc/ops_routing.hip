@@ -423,26 +423,57 @@ __device__ __forceinline__ int cost_group(int word) {
 // the number of pairs of expert e the wave has placed so far, base[e] where the wave's run starts.
 __device__ __forceinline__ void place_pairs(const int32_t* ids, int32_t* ids_dst, int E, int lo, int hi, int lane, int* next,
                                             const int* base) {
-    for (int first = lo; first < hi; first += 64) {
-        const int p = first + lane;
-        int e = -1;
-        if (p < hi) { e = ids[p]; if (static_cast<unsigned>(e) >= static_cast<unsigned>(E)) e = -1; }
-        unsigned long long remaining = __ballot(e >= 0);
-        int rank = 0, group = 0;
-        while (remaining) {
-            const int leader = __ffsll(static_cast<long long>(remaining)) - 1;
-            const int le = __shfl(e, leader, 64);
-            const unsigned long long same = __ballot(e == le);
-            if (e == le) {
-                rank = __popcll(same & ((1ull << lane) - 1ull));
-                group = __popcll(same);
-            }
-            remaining &= ~same;
+    // the ids of eight steps are requested together: a step is a dependent chain of ballots, and one round trip
+    // per step was most of the time this took
+    constexpr int kBatch = 8;
+    for (int first0 = lo; first0 < hi; first0 += 64 * kBatch) {
+        int loaded[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const int p = first0 + 64 * j + lane;
+            loaded[j] = p < hi ? ids[p] : -1;
         }
-        if (e >= 0) ids_dst[base[e] + next[e] + rank] = p;
-        __threadfence_block();
-        if (e >= 0 && rank == group - 1) next[e] += group;
-        __threadfence_block();
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const int first = first0 + 64 * j;
+            if (first >= hi) break;
+            const int p = first + lane;
+            int e = loaded[j];
+            if (static_cast<unsigned>(e) >= static_cast<unsigned>(E)) e = -1;
+            unsigned long long remaining = __ballot(e >= 0);
+            int rank = 0, group = 0;
+            while (remaining) {
+                const int leader = __ffsll(static_cast<long long>(remaining)) - 1;
+                const int le = __shfl(e, leader, 64);
+                const unsigned long long same = __ballot(e == le);
+                if (e == le) {
+                    rank = __popcll(same & ((1ull << lane) - 1ull));
+                    group = __popcll(same);
+                }
+                remaining &= ~same;
+            }
+            if (e >= 0) ids_dst[base[e] + next[e] + rank] = p;
+            __threadfence_block();
+            if (e >= 0 && rank == group - 1) next[e] += group;
+            __threadfence_block();
+        }
+    }
+}
+
+// Adds the ids of pairs [lo, hi) to the wave's histogram counts[E] (LDS).  The ids of a pass (16 per lane) are all
+// requested before the first is counted: one memory round trip per pass instead of one per 64 pairs.
+__device__ __forceinline__ void count_ids(const int32_t* ids, int E, int lo, int hi, int lane, int* counts) {
+    constexpr int kBatch = 16;
+    for (int first = lo; first < hi; first += 64 * kBatch) {
+        int loaded[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const int p = first + 64 * j + lane;
+            loaded[j] = p < hi ? ids[p] : -1;
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j)
+            if (static_cast<unsigned>(loaded[j]) < static_cast<unsigned>(E)) atomicAdd(&counts[loaded[j]], 1);
     }
 }
 
@@ -468,10 +499,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_scatter_kernel(PlanArgs a)
     wave_range(block_hi - block_lo, kWaves, wave, block_lo, lo, hi);
     for (int i = tid; i < kWaves * E; i += kPlanThreads) hist[i] = 0;
     __syncthreads();
-    for (int p = lo + lane; p < hi; p += 64) {
-        const int e = a.ids[p];
-        if (static_cast<unsigned>(e) < static_cast<unsigned>(E)) atomicAdd(&hist[wave * E + e], 1);
-    }
+    count_ids(a.ids, E, lo, hi, lane, hist + wave * E);
     __syncthreads();
     if (tid < E) {
         int before = a.wave_base[blockIdx.x * E + tid];
@@ -513,10 +541,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
     __syncthreads();
     int lo, hi;
     wave_range(a.pairs, kWaves, wave, 0, lo, hi);
-    for (int p = lo + lane; p < hi; p += 64) {
-        const int e = a.ids[p];
-        if (static_cast<unsigned>(e) < static_cast<unsigned>(E)) atomicAdd(&hist[wave * E + e], 1);
-    }
+    count_ids(a.ids, E, lo, hi, lane, hist + wave * E);
     __syncthreads();
     int count = 0;
     if (tid < E) {
