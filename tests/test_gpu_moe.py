@@ -90,9 +90,11 @@ def test_uniform_layer(uniform):
     assert rel_l2(out, oracle_layer(x, ids, weights, tensors)) <= FFN_TOL
 
 
-@pytest.mark.parametrize("hidden,inter", [(2048, 512), (640, 96), (1024, 32)])
+@pytest.mark.parametrize("hidden,inter", [(2048, 512), (640, 96), (1024, 32), (96, 64), (160, 128)])
 def test_decode_wide_rows(hidden, inter):
-    """Rows wider than 512 columns use 64 lanes per row; 640 leaves lanes without a column block."""
+    """Rows wider than 512 columns use 64 lanes per row; 640 leaves lanes without a column block.  The narrow shapes
+    have rows of two to eight groups: some classes then take their group levels as shared level words (at least
+    four levels per row) and some by one load per lane, in the same launch."""
     import torch
     from mfq_amd import runtime as R
     experts, k, tokens = 12, 4, 3
