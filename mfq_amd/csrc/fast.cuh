@@ -399,12 +399,11 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t b
     return d;
 }
 
-// fp16 bit pattern of the power of two `offset`, in both halves.
-__device__ constexpr uint32_t magic_pair(float offset) {
-    int exponent = 15;
-    for (float v = offset; v > 1.0f; v *= 0.5f) ++exponent;
-    return (static_cast<uint32_t>(exponent) << 10) * 0x00010001u;
-}
+// fp16 bit pattern of 2^LOG2, in both halves.  A template constant, not a function of a float: a loop over
+// floats is not folded by the compiler, and as a call it ran (ten iterations per use) inside the tile kernel's steps.
+template <int LOG2>
+constexpr uint32_t kMagicOf = (static_cast<uint32_t>(15 + LOG2) << 10) * 0x00010001u;
+static_assert(kMagicOf<10> == 0x64006400u, "1024.0 in both halves");
 
 // The fp16 pairs 4j .. 4j+3 of a lane block (NINT3, NINT4, NINT8, MXFP4): chunk j of the row.
 // MAGIC: integer codes as offset + q whatever the class (the tile kernel's form); otherwise as the row loop takes them.
@@ -426,10 +425,10 @@ __device__ __forceinline__ void chunk_pairs(const FastRaw<CLS>& raw, int j, uint
         if constexpr (kDenormal) {
             t[0] = w & 0x000f000fu; t[1] = w & 0x00f000f0u; t[2] = high & 0x000f000fu; t[3] = high & 0x00f000f0u;
         } else {
-            t[0] = and_or(w, 0x000f000fu, magic_pair(1024.0f));
-            t[1] = and_or(w, 0x00f000f0u, magic_pair(64.0f));
-            t[2] = and_or(high, 0x000f000fu, magic_pair(1024.0f));
-            t[3] = and_or(high, 0x00f000f0u, magic_pair(64.0f));
+            t[0] = and_or(w, 0x000f000fu, kMagicOf<10>);
+            t[1] = and_or(w, 0x00f000f0u, kMagicOf<6>);
+            t[2] = and_or(high, 0x000f000fu, kMagicOf<10>);
+            t[3] = and_or(high, 0x00f000f0u, kMagicOf<6>);
         }
     } else if constexpr (C::kBits == 8) {
         const uint32_t lo = raw.q[2 * j], hi = raw.q[2 * j + 1];
@@ -452,10 +451,10 @@ __device__ __forceinline__ void chunk_pairs(const FastRaw<CLS>& raw, int j, uint
         if constexpr (kDenormal) {
             t[0] = u & 0x00070007u; t[1] = u & 0x00380038u; t[2] = u & 0x01c001c0u; t[3] = (u >> 3) & 0x01c001c0u;
         } else {
-            t[0] = and_or(u, 0x00070007u, magic_pair(1024.0f));
-            t[1] = and_or(u, 0x00380038u, magic_pair(128.0f));
-            t[2] = and_or(u, 0x01c001c0u, magic_pair(16.0f));
-            t[3] = and_or(u >> 3, 0x01c001c0u, magic_pair(16.0f));
+            t[0] = and_or(u, 0x00070007u, kMagicOf<10>);
+            t[1] = and_or(u, 0x00380038u, kMagicOf<7>);
+            t[2] = and_or(u, 0x01c001c0u, kMagicOf<4>);
+            t[3] = and_or(u >> 3, 0x01c001c0u, kMagicOf<4>);
         }
     }
 }
@@ -764,10 +763,10 @@ __device__ __forceinline__ void chunk_weights(const WeightBlock<CLS>& k, const F
             // pairs 8d .. 8d+7 come from dword d: chunk j takes the (j % 2)-th four of dword j / 2
             const uint32_t word = raw.q[j / 2], high = word >> 8;
             const uint32_t from = (j % 2) ? high : word;
-            t[0] = and_or(from, 0x00030003u, magic_pair(1024.0f));
-            t[1] = and_or(from, 0x000c000cu, magic_pair(256.0f));
-            t[2] = and_or(from, 0x00300030u, magic_pair(64.0f));
-            t[3] = and_or(from, 0x00c000c0u, magic_pair(16.0f));
+            t[0] = and_or(from, 0x00030003u, kMagicOf<10>);
+            t[1] = and_or(from, 0x000c000cu, kMagicOf<8>);
+            t[2] = and_or(from, 0x00300030u, kMagicOf<6>);
+            t[3] = and_or(from, 0x00c000c0u, kMagicOf<4>);
         } else {
             chunk_pairs<CLS, true>(raw, j, t);
         }
