@@ -32,12 +32,11 @@ MFQ_HD LaneBlock lane_block(int cb, int width, int groups) {
     b.valid = cb * kLaneColumns < width;
     b.cb = b.valid ? cb : 0;
     b.group = (b.cb * kLaneColumns) / GS;
-    b.sel = 0;
-#if defined(__HIP_DEVICE_COMPILE__)
-#pragma unroll
-#endif
-    for (int j = 0; j < 4; ++j)
-        if ((b.cb * kLaneColumns + 8 * j) / GS != b.group) b.sel |= 1u << j;
+    // a lane block meets at most two groups (GS >= 16): chunk j lies in the second when it starts at or behind the
+    // group's end.  One remainder and four compares; a division per chunk is what the compiler made of the direct form.
+    static_assert(GS >= 16, "a lane block of 32 columns spans at most two groups");
+    const int rest = GS - (b.cb * kLaneColumns - b.group * GS);     // columns of the first group inside the block
+    b.sel = (8 >= rest ? 2u : 0u) | (16 >= rest ? 4u : 0u) | (24 >= rest ? 8u : 0u);
     // two consecutive levels come with one 16-bit load; the window slides back at the last group
     b.level_at = b.group < groups - 2 ? b.group : groups - 2;
     b.level_shift = 8 * (b.group - b.level_at);
