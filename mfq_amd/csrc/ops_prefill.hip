@@ -237,8 +237,17 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
     // of the row in LDS)
     const unsigned char* packed_row[MT];
     int packed_piece[MT];
+    // When no step meets a lane block behind the end of the row and the copy of the activations is below 4 GB, the
+    // copies take their address as a scalar base (layout + step) plus a 32-bit lane offset that never changes: no
+    // vector arithmetic per step.
+    const unsigned char* packed_base = nullptr;
+    uint32_t packed_offset[MT];
+    bool packed_scalar = false;
     if constexpr (PACKED) {
         const uint16_t* base = a.in_tiles + tile_layout<CLS>() * a.in_tiles_layout_stride;
+        packed_base = reinterpret_cast<const unsigned char*>(base);
+        const int64_t rows_in = a.in_per_pair ? a.pairs : (a.pairs + a.top_k - 1) / a.top_k;
+        packed_scalar = !ragged && rows_in * width * 2 < (int64_t(1) << 32);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const int r = 32 * i + 8 * wave + lane / 8;
@@ -246,9 +255,26 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
             const int64_t from = pair < 0 ? 0 : a.in_per_pair ? pair : pair / a.top_k;
             packed_row[i] = reinterpret_cast<const unsigned char*>(base + from * width);
             packed_piece[i] = (lane % 8) ^ tile_swizzle(r);
+            packed_offset[i] = static_cast<uint32_t>(from * width * 2 + packed_piece[i] * 16);
         }
     }
     auto x_direct = [&](int step) {
+        if (packed_scalar) {
+            // the same address in every lane; said so for the "s" operand below
+            const uintptr_t address = reinterpret_cast<uintptr_t>(packed_base + step * 128);
+            const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(address)));
+            const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(address >> 32)));
+            const unsigned char* from = reinterpret_cast<const unsigned char*>((static_cast<uintptr_t>(hi) << 32) | lo);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                unsigned char* to = x_lds + (step & 1) * kFastXBytes + (32 * i + 8 * wave) * 128;
+                const uint32_t lds_at = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
+                    reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)(to)))));
+                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                             :: "v"(packed_offset[i]), "s"(from), "s"(lds_at) : "memory", "m0");
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             int cb = 2 * step + packed_piece[i] / 4;
