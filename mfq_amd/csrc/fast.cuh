@@ -482,15 +482,6 @@ __device__ __forceinline__ uint32_t shift_add(uint32_t a, uint32_t b) {
     return d;
 }
 
-// Index k of the eight IB-bit indices in q, k not a template argument.
-template <int IB>
-__device__ __forceinline__ uint32_t nvq_index_at(const uint32_t (&q)[3], int k) {
-    const int bit = k * IB, word = bit >> 5, shift = bit & 31;
-    uint32_t v = q[word] >> shift;
-    if (shift + IB > 32) v |= q[word + 1] << (32 - shift);
-    return v & ((1u << IB) - 1u);
-}
-
 // Index K of the eight IB-bit indices in q.
 template <int IB, int K>
 __device__ __forceinline__ uint32_t nvq_index(const uint32_t (&q)[3]) {
@@ -697,8 +688,8 @@ struct WeightBlock {
     uint32_t sel;                        // bit j: chunk j belongs to the block's second group
     half2_t level[2], shift[2];          // NINT: per group, both halves equal
     half2_t scale[2];                    // NVQ: multiplier of the state of each group
-    const unsigned char* bank[2];        // NVQ: codebook bank of each group (LDS)
-    const unsigned char* signs;          // NVQ: sign table (LDS)
+    uint32_t bank_at[2];                 // NVQ: LDS byte address of the codebook bank of each group
+    uint32_t signs_at;                   // NVQ: LDS byte address of the sign table
     uint32_t masks;                      // NVQ: the four 7-bit sign masks
     uint32_t q2;                         // NVQ: third index word, aligned
     float block_scale;                   // MXFP4: 2^(s-127)
@@ -719,9 +710,10 @@ __device__ __forceinline__ WeightBlock<CLS> weight_block(const FastCtx<CLS>& c, 
         const uint32_t state0 = states & 15u, state1 = (states >> 4) & 15u;
         k.scale[0] = splat_half(c.multiplier[state0]);
         k.scale[1] = splat_half(c.multiplier[state1]);
-        k.bank[0] = c.codebook + c.bank_byte[state0];
-        k.bank[1] = c.codebook + c.bank_byte[state1];
-        k.signs = c.signs;
+        typedef const __attribute__((address_space(3))) unsigned char* lds_bytes;
+        k.bank_at[0] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_bytes)(c.codebook + c.bank_byte[state0])));
+        k.bank_at[1] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_bytes)(c.codebook + c.bank_byte[state1])));
+        k.signs_at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_bytes)c.signs));
     } else if constexpr (C::kMx) {
         k.block_scale = bits_to_float(raw.a ? (raw.a << 23) : 0x00400000u);
     } else {
@@ -741,16 +733,27 @@ template <int CLS, int IB>
 __device__ __forceinline__ void chunk_weights(const WeightBlock<CLS>& k, const FastRaw<CLS>& raw, int j, uint32_t (&w)[4]) {
     using C = FastClass<CLS>;
     if constexpr (C::kNvq) {
+        static_assert(C::kGs == 24, "the first chunk of a lane block lies in its first group, the last in its second");
         const uint32_t q[3] = {raw.q[0], raw.q[1], k.q2};
-        const bool second = (k.sel >> j) & 1u;
-        const unsigned char* bank = second ? k.bank[1] : k.bank[0];
-        const u32x2 lo = *reinterpret_cast<const u32x2*>(bank + 8 * nvq_index_at<IB>(q, 2 * j));
-        const u32x2 hi = *reinterpret_cast<const u32x2*>(bank + 8 * nvq_index_at<IB>(q, 2 * j + 1));
-        const u32x4 sign = *reinterpret_cast<const u32x4*>(k.signs + 16 * ((k.masks >> (7 * j)) & 127u));
-        const uint32_t t[4] = {lo[0] ^ sign[0], lo[1] ^ sign[1], hi[0] ^ sign[2], hi[1] ^ sign[3]};
-        const half2_t scale = second ? k.scale[1] : k.scale[0];
+        // the chunk as a compile-time constant: index fields and LDS addresses each as the one instruction the hardware has
+        auto chunk = [&](auto jc) {
+            constexpr int J = decltype(jc)::value;
+            const bool second = J == 0 ? false : J == 3 ? true : ((k.sel >> J) & 1u) != 0;
+            const uint32_t bank = second ? k.bank_at[1] : k.bank_at[0];
+            typedef const __attribute__((address_space(3))) u32x2* lds2;
+            typedef const __attribute__((address_space(3))) u32x4* lds4;
+            const u32x2 lo = *(lds2)(uintptr_t)shift_add<3>(nvq_index<IB, 2 * J>(q), bank);
+            const u32x2 hi = *(lds2)(uintptr_t)shift_add<3>(nvq_index<IB, 2 * J + 1>(q), bank);
+            const u32x4 sign = *(lds4)(uintptr_t)shift_add<4>(bit_field<7 * J, 7>(k.masks), k.signs_at);
+            const uint32_t t[4] = {lo[0] ^ sign[0], lo[1] ^ sign[1], hi[0] ^ sign[2], hi[1] ^ sign[3]};
+            const half2_t scale = second ? k.scale[1] : k.scale[0];
 #pragma unroll
-        for (int m = 0; m < 4; ++m) w[m] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, t[m]) * scale);
+            for (int m = 0; m < 4; ++m) w[m] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, t[m]) * scale);
+        };
+        if (j == 0) chunk(std::integral_constant<int, 0>{});
+        else if (j == 1) chunk(std::integral_constant<int, 1>{});
+        else if (j == 2) chunk(std::integral_constant<int, 2>{});
+        else chunk(std::integral_constant<int, 3>{});
     } else if constexpr (C::kMx) {
         w[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(raw.q[j], k.block_scale, 0));
         w[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(raw.q[j], k.block_scale, 1));
