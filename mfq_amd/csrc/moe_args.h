@@ -79,9 +79,6 @@ void launch_tiles_mx_scaled(const RowsArgs& args, int slots, int max_tiles, hipS
 void launch_fp8_split(const void* src, int dtype, int rows, int width, int terms, uint8_t* dst, uint8_t* scales, hipStream_t stream);
 // Pair layout (0..3) in which the streaming tile kernel reads the activations of a pool of this class.
 int tile_layout_of_class(int cls);
-// dst[layout][rows][width] = fp16 copy of src (fp16 or bf16) in the pair order of every layout in the mask.
-void launch_tile_pack(const void* src, int dtype, int rows, int width, uint32_t layouts, uint16_t* dst, int64_t layout_stride,
-                      hipStream_t stream);
 // SwiGLU whose output rows are in the pair order their down projection reads (down_info: [experts]).
 void launch_swiglu_tiles(const uint16_t* gate, const uint16_t* up, int64_t gate_stride, int inner, int pairs, float limit,
                          const uint16_t* table, const int32_t* ids, const ExpertInfo* down_info, int experts, uint16_t* hidden,

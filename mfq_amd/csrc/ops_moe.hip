@@ -857,6 +857,15 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
             plan.pack.vector_ok = reinterpret_cast<uintptr_t>(x_dev) % 16 == 0 &&
                                   (static_cast<int64_t>(H) * (f->config.x_dtype == MFQ_AMD_F32 ? 4 : 2)) % 16 == 0;
         }
+        // prefill: the fp16 copies of the activations in the pair layouts of the tile kernel are made by the spare
+        // blocks of the plan kernel (the plan itself keeps one CU busy)
+        const int x_element = f->config.x_dtype == MFQ_AMD_F32 ? 4 : 2;
+        const bool x_vector_ok = reinterpret_cast<uintptr_t>(x_dev) % 16 == 0 && (static_cast<int64_t>(H) * x_element) % 16 == 0;
+        const bool x_tiles = !decode && f->d_x_tiles != nullptr && tiles_fast_geometry(H, f->config.x_dtype, x_vector_ok);
+        if (x_tiles) {
+            plan.tiles.src = x_dev; plan.tiles.dst = f->d_x_tiles; plan.tiles.layout_stride = static_cast<int64_t>(tokens) * H;
+            plan.tiles.rows = tokens; plan.tiles.width = H; plan.tiles.dtype = f->config.x_dtype; plan.tiles.layouts = f->x_tile_layouts;
+        }
         f->mark(0, stream);
         if (route != nullptr) plan.route = *route;
         launch_route_plan(plan, stream);
@@ -943,11 +952,7 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         rows.out = f->d_gu; rows.out_pair_stride = 2 * static_cast<int64_t>(I); rows.out_slot_stride = I;
         rows.slot_base = 0; rows.out_rows = I;
         rows.in_packed = pack_x ? f->d_x_packed : nullptr; rows.in_packed_stride = dev::xpack_row_dwords(H);
-        if (!decode && f->d_x_tiles != nullptr && tiles_fast_geometry(H, rows.in_dtype, rows.in_vector_ok)) {
-            const int64_t layout_stride = static_cast<int64_t>(tokens) * H;
-            launch_tile_pack(x_dev, rows.in_dtype, tokens, H, f->x_tile_layouts, f->d_x_tiles, layout_stride, stream);
-            rows.in_tiles = f->d_x_tiles; rows.in_tiles_layout_stride = layout_stride;
-        }
+        if (x_tiles) { rows.in_tiles = f->d_x_tiles; rows.in_tiles_layout_stride = static_cast<int64_t>(tokens) * H; }
         run_rows(0, 2);
         f->mark(2, stream);
 

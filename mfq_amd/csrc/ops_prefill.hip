@@ -19,6 +19,7 @@
 #include "fp8_split.h"
 #include "launch.cuh"
 #include "moe_args.h"
+#include "tile_pack.cuh"
 #include "xpack.cuh"
 
 namespace mfq_amd {
@@ -144,31 +145,10 @@ __device__ __forceinline__ half8_t as_half8(uint32_t a, uint32_t b, uint32_t c, 
     return __builtin_bit_cast(half8_t, u32x4{a, b, c, d});
 }
 
-// Which of the four fp16 copies of the activations (tile_pack_kernel, swiglu_tiles_kernel) a class reads: the
+// Which of the four fp16 copies of the activations (the spare blocks of route_plan_kernel, swiglu_tiles_kernel) a class reads: the
 // pair order of its weights, without the powers of two the row loop's packed form carries.
 template <int CLS> __host__ __device__ constexpr int tile_layout() {
     return CLS == K_NINT_8_48 ? 1 : (CLS == K_NVQ_D4 || CLS == K_MXFP4) ? 2 : CLS == K_NINT_2_16 ? 3 : 0;
-}
-
-// Converts 32 consecutive activations (64 bytes as loaded) to the 16 fp16 pairs of the class.
-template <int CLS, bool HALF>
-__device__ __forceinline__ void x_pairs(const u32x4 (&raw)[4], uint32_t (&p)[16]) {
-    const uint32_t words[16] = {raw[0][0], raw[0][1], raw[0][2], raw[0][3], raw[1][0], raw[1][1], raw[1][2], raw[1][3],
-                                raw[2][0], raw[2][1], raw[2][2], raw[2][3], raw[3][0], raw[3][1], raw[3][2], raw[3][3]};
-#pragma unroll
-    for (int k = 0; k < 16; ++k) {
-        const int first = pair_column<CLS>(k, 0), second = pair_column<CLS>(k, 1);
-        if (HALF) {
-            // select two of the four halves of two words: one byte permute
-            const uint32_t selector = ((first & 1) ? 0x0302u : 0x0100u) | ((second & 1) ? 0x07060000u : 0x05040000u);
-            p[k] = __builtin_amdgcn_perm(words[second / 2], words[first / 2], selector);
-        } else {
-            // bf16 -> fp32 is a shift; values inside the fp16 range convert without rounding
-            const uint32_t a = (first & 1) ? words[first / 2] & 0xffff0000u : words[first / 2] << 16;
-            const uint32_t b = (second & 1) ? words[second / 2] & 0xffff0000u : words[second / 2] << 16;
-            p[k] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bits_to_float(a), bits_to_float(b)));
-        }
-    }
 }
 
 // Loads per call of fast_fetch without the NINT levels and the NVQ side streams (vector memory instructions), for
@@ -184,7 +164,7 @@ constexpr int fetch_loads() {
 // (same c, consecutive rows) over all banks.
 __device__ __forceinline__ int tile_swizzle(int row) { return ((row & 7) + (row >> 3)) & 7; }
 
-// PACKED: the activations come as fp16 in the pair order of the class (tile_pack_kernel,
+// PACKED: the activations come as fp16 in the pair order of the class (spare blocks of route_plan_kernel,
 // swiglu_tiles_kernel) and go to LDS by direct loads; otherwise they are converted in the kernel.
 template <int CLS, int MT, int IB, bool PACKED>
 __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, int row_block, int pool_index, int local, int begin,
@@ -798,42 +778,6 @@ __global__ void __launch_bounds__(256) fp8_split_kernel(const uint16_t* src, int
 
 
 // ------------------------------------------------ activations for the tiles ----
-// The four pair layouts of tile_layout<CLS>() as classes that have them.
-template <int LAYOUT> struct LayoutClass;
-template <> struct LayoutClass<0> { static constexpr int value = K_NINT_4_24; };
-template <> struct LayoutClass<1> { static constexpr int value = K_NINT_8_48; };
-template <> struct LayoutClass<2> { static constexpr int value = K_NVQ_D4; };
-template <> struct LayoutClass<3> { static constexpr int value = K_NINT_2_16; };
-
-template <int LAYOUT>
-__device__ __forceinline__ void store_layout(const u32x4 (&raw)[4], bool half_in, uint16_t* dst) {
-    uint32_t p[16];
-    if (half_in) x_pairs<LayoutClass<LAYOUT>::value, true>(raw, p);
-    else x_pairs<LayoutClass<LAYOUT>::value, false>(raw, p);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-        *reinterpret_cast<u32x4*>(dst + 8 * j) = u32x4{p[4 * j], p[4 * j + 1], p[4 * j + 2], p[4 * j + 3]};
-}
-
-// dst[layout][row][width] = fp16(src[row][width]) with every 32 columns in the pair order of the layout,
-// for the layouts in the mask.  One thread per lane block.
-__global__ void __launch_bounds__(256) tile_pack_kernel(const void* src, int dtype, int rows, int width, uint32_t layouts,
-                                                        uint16_t* dst, int64_t layout_stride) {
-    const int blocks = width / kLaneColumns;
-    const int64_t item = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (item >= static_cast<int64_t>(rows) * blocks) return;
-    const unsigned char* from = static_cast<const unsigned char*>(src) + item * 64;
-    u32x4 raw[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) raw[j] = *(const MFQ_GLOBAL u32x4*)(from + 16 * j);
-    const bool half_in = dtype == MFQ_AMD_F16;
-    uint16_t* to = dst + item * kLaneColumns;
-    if (layouts & 1u) store_layout<0>(raw, half_in, to);
-    if (layouts & 2u) store_layout<1>(raw, half_in, to + layout_stride);
-    if (layouts & 4u) store_layout<2>(raw, half_in, to + 2 * layout_stride);
-    if (layouts & 8u) store_layout<3>(raw, half_in, to + 3 * layout_stride);
-}
-
 // hidden[pair] = swiglu(gate[pair], up[pair]) as fp16, every 32 columns in the pair order that the
 // pair's down projection reads: the layout of its pool's class when the streaming tile kernel serves
 // the pool, plain column order otherwise (which is also layout 2).  One thread per lane block.
@@ -967,16 +911,6 @@ void launch_fp8_split(const void* src, int dtype, int rows, int width, int terms
     hipLaunchKernelGGL(dev::fp8_split_kernel, dim3(static_cast<unsigned>((items + 255) / 256)), dim3(256), 0, stream,
                        static_cast<const uint16_t*>(src), dtype == MFQ_AMD_F16 ? 1 : 0, items, width, terms, dst, scales);
     check_launch("fp8_split_kernel");
-}
-
-void launch_tile_pack(const void* src, int dtype, int rows, int width, uint32_t layouts, uint16_t* dst, int64_t layout_stride,
-                      hipStream_t stream) {
-    if (rows <= 0 || layouts == 0) return;
-    MFQ_REQUIRE(width % dev::kLaneColumns == 0 && dtype != MFQ_AMD_F32, "geometry is not served by the tile pack kernel");
-    const int64_t items = static_cast<int64_t>(rows) * (width / dev::kLaneColumns);
-    hipLaunchKernelGGL(dev::tile_pack_kernel, dim3(static_cast<unsigned>((items + 255) / 256)), dim3(256), 0, stream, src, dtype,
-                       rows, width, layouts, dst, layout_stride);
-    check_launch("tile_pack_kernel");
 }
 
 void launch_swiglu_tiles(const uint16_t* gate, const uint16_t* up, int64_t gate_stride, int inner, int pairs, float limit,

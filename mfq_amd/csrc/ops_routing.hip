@@ -3,6 +3,7 @@
 #include "decode.cuh"
 #include "device_state.h"
 #include "plan.h"
+#include "tile_pack.cuh"
 #include "xpack.cuh"
 
 namespace mfq_amd {
@@ -518,6 +519,12 @@ __global__ void __launch_bounds__(kPlanThreads) route_scatter_kernel(PlanArgs a)
 // same expert rank themselves by ballot, so compact slots keep ascending pair order.
 __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
     extern __shared__ int lds[];
+    if (blockIdx.x > 0 && a.tiles.src != nullptr) {
+        // blocks behind the first copy the activations into the pair layouts of the tile kernel while the first builds the plan
+        const int64_t item = static_cast<int64_t>(blockIdx.x - 1) * kPlanThreads + threadIdx.x;
+        tile_pack_item(item, a.tiles.src, a.tiles.dtype, a.tiles.rows, a.tiles.width, a.tiles.layouts, a.tiles.dst, a.tiles.layout_stride);
+        return;
+    }
     if (blockIdx.x > 0) {
         // blocks behind the first pack one activation row each while the first builds the plan
         const int row = blockIdx.x - 1;
@@ -1136,6 +1143,8 @@ void launch_route_plan(const PlanArgs& args, hipStream_t stream) {
                     (args.pairs <= kPlanThreads && args.extras.items != nullptr && args.extras.expert_info != nullptr &&
                      args.extras.pair_items != nullptr && !args.extras.want_tiles && !args.extras.want_items),
                 "pair records in pair order need a decode-sized plan with resolved expert records and no other lists");
+    const bool large = !args.extras.pairs_only && !(args.pairs <= kPlanThreads && (args.extras.items == nullptr || !args.extras.want_tiles));
+    MFQ_REQUIRE(args.tiles.src == nullptr || large, "only the large plan kernel copies activations into the tile layouts");
     if (args.extras.pairs_only) {
         MFQ_REQUIRE(args.pairs <= kPlanSortPairs && args.extras.expert_words != nullptr && args.extras.pair_items != nullptr &&
                         !args.extras.want_tiles && !args.extras.want_items && args.extras.slots >= 1 && args.extras.slots <= kSlots,
@@ -1175,7 +1184,15 @@ void launch_route_plan(const PlanArgs& args, hipStream_t stream) {
     }
     MFQ_REQUIRE(args.route.logits == nullptr, "fused routing needs a decode-sized plan");
     MFQ_REQUIRE(args.wave_base == nullptr || args.extras.pair_items == nullptr, "per-pair records need the one-kernel plan");
-    hipLaunchKernelGGL(dev::route_plan_kernel, dim3(1 + pack_rows), dim3(kPlanThreads), lds, stream, args);
+    int spare_blocks = pack_rows;
+    if (args.tiles.src != nullptr) {
+        MFQ_REQUIRE(pack_rows == 0 && args.tiles.dst != nullptr && args.tiles.width % dev::kLaneColumns == 0 && args.tiles.dtype != MFQ_AMD_F32 &&
+                        reinterpret_cast<uintptr_t>(args.tiles.src) % 16 == 0,
+                    "activations cannot be copied into the tile layouts by the plan kernel");
+        const int64_t items = static_cast<int64_t>(args.tiles.rows) * (args.tiles.width / dev::kLaneColumns);
+        spare_blocks = static_cast<int>((items + kPlanThreads - 1) / kPlanThreads);
+    }
+    hipLaunchKernelGGL(dev::route_plan_kernel, dim3(1 + spare_blocks), dim3(kPlanThreads), lds, stream, args);
     check_launch("route_plan_kernel");
     if (args.wave_base != nullptr) {
         const size_t scatter_lds = sizeof(int) * 2 * (kPlanThreads / 64) * args.experts;

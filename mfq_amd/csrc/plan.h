@@ -97,6 +97,16 @@ struct PlanPack {
     int32_t rows, width, dtype, vector_ok;
 };
 
+// Activation rows to copy as fp16 in the pair layouts of the streaming tile kernel (prefill): the spare blocks of the
+// large plan kernel do it, kPlanThreads lane blocks of 32 columns each.
+struct PlanTilePack {
+    const void* src;        // [rows][width] activations (fp16 or bf16, 16-byte aligned rows), null = nothing to copy
+    uint16_t* dst;          // [4][rows][width]: the copies, layout_stride halves apart
+    int64_t layout_stride;
+    int32_t rows, width, dtype;
+    uint32_t layouts;       // bit l: layout l is wanted
+};
+
 // Router logits to select the routes from inside the plan kernel (decode only), or logits == null.
 struct PlanRoute {
     const void* logits;       // [tokens, experts]
@@ -119,6 +129,7 @@ struct PlanArgs {
                               // one-thread-per-pair kernel places its pairs with a second, multi-block kernel
     PlanExtras extras;        // extras.items == nullptr: plain route plan
     PlanPack pack;
+    PlanTilePack tiles;
     PlanRoute route;
 };
 
