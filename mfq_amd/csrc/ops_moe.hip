@@ -622,8 +622,8 @@ struct mfq_amd_moe_ffn {
     ExpertInfo* d_expert_info = nullptr;
     uint32_t* d_expert_words = nullptr;
     int32_t *d_expert_pool = nullptr, *d_items = nullptr, *d_class_offsets = nullptr, *d_tile_items = nullptr,
-            *d_tile_offsets = nullptr, *d_counts = nullptr, *d_bounds = nullptr, *d_tile_bounds = nullptr,
-            *d_tile_experts = nullptr, *d_ids_dst = nullptr, *d_distinct = nullptr;
+            *d_tile_offsets = nullptr, *d_counts = nullptr, *d_bounds = nullptr,
+            *d_ids_dst = nullptr, *d_distinct = nullptr;
     int64_t* d_touched = nullptr;
     uint16_t *d_gu = nullptr, *d_hidden = nullptr, *d_pairs = nullptr;
     const uint16_t* d_sigmoid = nullptr;   // the device's table: not owned
@@ -653,7 +653,7 @@ struct mfq_amd_moe_ffn {
 
     ~mfq_amd_moe_ffn() {
         void* all[] = {d_pools, d_pool_class, d_pool_bytes, d_expert_pool, d_expert_info, d_expert_words, d_item_info, d_pair_items, d_items, d_class_offsets, d_tile_items,
-                       d_tile_offsets, d_counts, d_bounds, d_tile_bounds, d_tile_experts, d_ids_dst, d_distinct,
+                       d_tile_offsets, d_counts, d_bounds, d_ids_dst, d_distinct,
                        d_touched, d_gu, d_hidden, d_pairs, d_logits, d_x_packed, d_hidden_packed, d_route_ids, d_route_weights, d_x_tiles, d_wave_base, d_fp8, d_fp8_scales,
                        d_shared_ids, d_shared_weights, d_shared_out};
         for (void* p : all) if (p) (void)hipFree(p);
@@ -757,8 +757,6 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
         f->d_tile_offsets = device_alloc<int32_t>(kSlots * kClassSlots);
         f->d_counts = device_alloc<int32_t>(E);
         f->d_bounds = device_alloc<int32_t>(E + 1);
-        f->d_tile_bounds = device_alloc<int32_t>(E + 1);
-        f->d_tile_experts = device_alloc<int32_t>(pairs / 8 + E + 1);
         f->d_ids_dst = device_alloc<int32_t>(pairs);
         f->d_distinct = device_alloc<int32_t>(1);
         f->d_touched = device_alloc<int64_t>(1);
@@ -826,8 +824,7 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         plan.ids = ids_dev; plan.pairs = pairs; plan.experts = E; plan.tile_m = 8; plan.top_k = k;
         plan.counts = f->d_counts; plan.expert_bounds = f->d_bounds; plan.ids_dst = f->d_ids_dst;
         // the per-8-route tile lists of the reference plan are not consumed by the decode kernels
-        plan.tile_bounds = decode ? nullptr : f->d_tile_bounds;
-        plan.tile_experts = decode ? nullptr : f->d_tile_experts;
+        // (the route tile tables of mfq_amd_route_plan are not asked for: the kernels here walk tile_items)
         plan.wave_base = !decode && pairs > 4 * kPlanThreads ? f->d_wave_base : nullptr;
         auto& x = plan.extras;
         x.pools = f->d_pools; x.pool_class = f->d_pool_class; x.pool_bytes = f->d_pool_bytes;
@@ -1158,7 +1155,7 @@ extern "C" void mfq_amd_moe_ffn_destroy(mfq_amd_moe_ffn* f) { delete f; }
 namespace {
 struct GroupedLayout {
     int64_t pools, pool_class, pool_bytes, expert_pool, items, item_info, pair_items, class_offsets, tile_items, tile_offsets, counts, bounds,
-            tile_bounds, tile_experts, ids_dst, touched, distinct, total;
+            ids_dst, touched, distinct, total;
     int tile_capacity;
 };
 GroupedLayout grouped_layout(int tokens, int top_k, int experts) {
@@ -1179,8 +1176,6 @@ GroupedLayout grouped_layout(int tokens, int top_k, int experts) {
     g.tile_offsets = take(4 * kClassSlots);
     g.counts = take(4 * experts);
     g.bounds = take(4 * (experts + 1));
-    g.tile_bounds = take(4 * (experts + 1));
-    g.tile_experts = take(4 * (pairs / 8 + experts + 1));
     g.ids_dst = take(4 * (pairs + 1));
     g.touched = take(8);
     g.distinct = take(4);
@@ -1244,8 +1239,6 @@ void grouped_matmul(const mfq_amd_moe_tensor* tensor, const void* x_dev, int32_t
         plan.ids = ids_dev; plan.pairs = pairs; plan.experts = E; plan.tile_m = 8; plan.top_k = top_k;
         plan.counts = reinterpret_cast<int32_t*>(at(g.counts));
         plan.expert_bounds = reinterpret_cast<int32_t*>(at(g.bounds));
-        plan.tile_bounds = reinterpret_cast<int32_t*>(at(g.tile_bounds));
-        plan.tile_experts = reinterpret_cast<int32_t*>(at(g.tile_experts));
         plan.ids_dst = reinterpret_cast<int32_t*>(at(g.ids_dst));
         auto& x = plan.extras;
         x.pools = reinterpret_cast<const mfq_amd_projection*>(at(g.pools));
