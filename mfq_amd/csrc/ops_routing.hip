@@ -630,21 +630,25 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
             if (lane == 0) { wave_items[c * kWaves + wave] = __popcll(mask); wave_tiles[c * kWaves + wave] = wave_total; }
         }
         __syncthreads();
-        if (tid == 0) {
-            int items_before = 0, tiles_before = 0;
-            for (int c = 0; c < K_CLASS_COUNT; ++c) {
-                x.class_offsets[s * kClassSlots + c] = items_before;
-                x.tile_offsets[s * kClassSlots + c] = tiles_before;
-                for (int w = 0; w < kWaves; ++w) {
-                    const int n = wave_items[c * kWaves + w], t = wave_tiles[c * kWaves + w];
-                    wave_items[c * kWaves + w] = items_before;
-                    wave_tiles[c * kWaves + w] = tiles_before;
-                    items_before += n;
-                    tiles_before += t;
+        {
+            // exclusive prefix over the (class, wave) cells in class-major order, as two block scans
+            constexpr int kCells = K_CLASS_COUNT * kWaves;
+            static_assert(kCells <= kPlanThreads, "one thread per (class, wave) cell");
+            const int n = tid < kCells ? wave_items[tid] : 0, t = tid < kCells ? wave_tiles[tid] : 0;
+            const int items_through = block_inclusive_scan(n, scratch);
+            const int tiles_through = block_inclusive_scan(t, scratch);
+            if (tid < kCells) {
+                wave_items[tid] = items_through - n;
+                wave_tiles[tid] = tiles_through - t;
+                if (tid % kWaves == 0) {
+                    x.class_offsets[s * kClassSlots + tid / kWaves] = items_through - n;
+                    x.tile_offsets[s * kClassSlots + tid / kWaves] = tiles_through - t;
+                }
+                if (tid == kCells - 1) {
+                    x.class_offsets[s * kClassSlots + K_CLASS_COUNT] = items_through;
+                    x.tile_offsets[s * kClassSlots + K_CLASS_COUNT] = tiles_through;
                 }
             }
-            x.class_offsets[s * kClassSlots + K_CLASS_COUNT] = items_before;
-            x.tile_offsets[s * kClassSlots + K_CLASS_COUNT] = tiles_before;
         }
         __syncthreads();
         if (my_class >= 0) {
