@@ -385,6 +385,11 @@ __global__ void __launch_bounds__(64) topk_kernel(const void* logits, int dtype,
 }
 
 // -------------------------------------------------------- route plan ----
+// Barrier for data the block exchanges through LDS only: a wave waits for its own LDS operations, not for its global
+// stores.  (__syncthreads() is also a fence for global memory: every wave first waits until each of its stores has
+// been acknowledged, about a microsecond wherever stores precede it.)
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 __device__ __forceinline__ int block_inclusive_scan(int value, int* wave_totals) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
@@ -392,9 +397,9 @@ __device__ __forceinline__ int block_inclusive_scan(int value, int* wave_totals)
         const int other = __shfl_up(value, offset, 64);
         if (lane >= offset) value += other;
     }
-    __syncthreads();
+    lds_barrier();
     if (lane == 63) wave_totals[wave] = value;
-    __syncthreads();
+    lds_barrier();
     int prefix = 0;
     for (int w = 0; w < wave; ++w) prefix += wave_totals[w];
     return value + prefix;
@@ -545,11 +550,11 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
     for (int i = tid; i < kWaves * E; i += kPlanThreads) hist[i] = 0;
-    __syncthreads();
+    lds_barrier();
     int lo, hi;
     wave_range(a.pairs, kWaves, wave, 0, lo, hi);
     count_ids(a.ids, E, lo, hi, lane, hist + wave * E);
-    __syncthreads();
+    lds_barrier();
     int count = 0;
     if (tid < E) {
         for (int w = 0; w < kWaves; ++w) { const int c = hist[w * E + tid]; hist[w * E + tid] = count; count += c; }
@@ -569,7 +574,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
         }
     }
     if (tid == 0) { a.expert_bounds[0] = 0; if (want_route_tiles) a.tile_bounds[0] = 0; }
-    __syncthreads();
+    lds_barrier();
 
     if (a.wave_base != nullptr) {
         // the pairs are placed by route_scatter_kernel, one block per wave range of this kernel
@@ -584,7 +589,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
     // Work lists per slot: active experts ordered by (kernel class, expert id), and their prefill
     // tiles in the same order.  Ranks come from per-class ballots inside a wave plus a small table
     // of per-(class, wave) totals.
-    __syncthreads();
+    lds_barrier();
     int* total_distinct = totals;
     unsigned long long* total_bytes = reinterpret_cast<unsigned long long*>(
         lds + ((totals + 2 - lds + 1) & ~1));                 // 8-byte aligned slot behind the counters
@@ -593,7 +598,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
     if (tid == 0) { *total_bytes = 0ull; *total_distinct = 0; }
     unsigned long long my_bytes = 0ull;
     for (int s = 0; s < x.slots; ++s) {
-        __syncthreads();
+        lds_barrier();
         int my_pool = -1;
         ExpertInfo info{-1, 0, -1, 0, 0};
         if (tid < E) {
@@ -629,7 +634,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
             const int wave_total = __shfl(scan, 63, 64);
             if (lane == 0) { wave_items[c * kWaves + wave] = __popcll(mask); wave_tiles[c * kWaves + wave] = wave_total; }
         }
-        __syncthreads();
+        lds_barrier();
         {
             // exclusive prefix over the (class, wave) cells in class-major order, as two block scans
             constexpr int kCells = K_CLASS_COUNT * kWaves;
@@ -650,7 +655,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();
         if (my_class >= 0) {
             const int at = s * E + wave_items[my_class * kWaves + wave] + my_rank;
             x.items[at] = tid;
