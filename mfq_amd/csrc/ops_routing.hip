@@ -385,6 +385,18 @@ __global__ void __launch_bounds__(64) topk_kernel(const void* logits, int dtype,
 }
 
 // -------------------------------------------------------- route plan ----
+// Inclusive prefix sum over the 64 lanes of a wave with data-parallel-primitive moves (shifts inside rows of 16 lanes,
+// then the last lane of a row broadcast to the rows behind it): six adds, no LDS traffic as the lane shuffles have.
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);    // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);    // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);    // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);    // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);    // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);    // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 // Barrier for data the block exchanges through LDS only: a wave waits for its own LDS operations, not for its global
 // stores.  (__syncthreads() is also a fence for global memory: every wave first waits until each of its stores has
 // been acknowledged, about a microsecond wherever stores precede it.)
@@ -392,11 +404,7 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 
 __device__ __forceinline__ int block_inclusive_scan(int value, int* wave_totals) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-    for (int offset = 1; offset < 64; offset <<= 1) {
-        const int other = __shfl_up(value, offset, 64);
-        if (lane >= offset) value += other;
-    }
+    value = wave_inclusive_scan(value);
     lds_barrier();
     if (lane == 63) wave_totals[wave] = value;
     lds_barrier();
@@ -621,17 +629,12 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
         for (int c = 0; c < K_CLASS_COUNT; ++c) {
             const bool flag = my_class == c;
             const unsigned long long mask = __ballot(flag);
-            int scan = flag ? my_tiles : 0;
-#pragma unroll
-            for (int offset = 1; offset < 64; offset <<= 1) {
-                const int other = __shfl_up(scan, offset, 64);
-                if (lane >= offset) scan += other;
-            }
+            const int scan = wave_inclusive_scan(flag ? my_tiles : 0);
             if (flag) {
                 my_rank = __popcll(mask & ((1ull << lane) - 1ull));
                 my_tile_rank = scan - my_tiles;
             }
-            const int wave_total = __shfl(scan, 63, 64);
+            const int wave_total = __builtin_amdgcn_readlane(scan, 63);
             if (lane == 0) { wave_items[c * kWaves + wave] = __popcll(mask); wave_tiles[c * kWaves + wave] = wave_total; }
         }
         lds_barrier();
