@@ -498,102 +498,16 @@ __device__ __forceinline__ void wave_range(int pairs, int waves, int wave, int b
     hi = lo + per_wave < begin + pairs ? lo + per_wave : begin + pairs;
 }
 
-// Second kernel of a large plan: block b places the pairs of wave range b of route_plan_kernel, split
-// again over its own waves; wave_base[b][e] (written by route_plan_kernel) is where the block's run of
-// expert e starts.
-__global__ void __launch_bounds__(kPlanThreads) route_scatter_kernel(PlanArgs a) {
-    extern __shared__ int lds[];
+// Work lists of a plan per slot: active experts ordered by (kernel class, expert id), their prefill tiles in the same
+// order, the per-pair records where asked for, and the byte and expert totals.  One block of kPlanThreads threads;
+// cnt[e], start[e] (LDS) hold the pairs of expert e and where they begin in ids_dst.  scratch [kWaves], wave_items and
+// wave_tiles [K_CLASS_COUNT][kWaves], totals [8] are LDS work arrays; lds is the base of the block's dynamic LDS.
+__device__ __forceinline__ void plan_work_lists(const PlanArgs& a, int* lds, int* cnt, int* start, int* scratch, int* wave_items,
+                                                int* wave_tiles, int* totals) {
     const int E = a.experts;
     constexpr int kWaves = kPlanThreads / 64;
-    int* hist = lds;                    // [kWaves][E]: counts, then pairs placed so far
-    int* base = hist + kWaves * E;      // [kWaves][E]: start of the run of (wave, expert)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    int block_lo, block_hi, lo, hi;
-    wave_range(a.pairs, kWaves, blockIdx.x, 0, block_lo, block_hi);
-    wave_range(block_hi - block_lo, kWaves, wave, block_lo, lo, hi);
-    for (int i = tid; i < kWaves * E; i += kPlanThreads) hist[i] = 0;
-    __syncthreads();
-    count_ids(a.ids, E, lo, hi, lane, hist + wave * E);
-    __syncthreads();
-    if (tid < E) {
-        int before = a.wave_base[blockIdx.x * E + tid];
-        for (int w = 0; w < kWaves; ++w) {
-            base[w * E + tid] = before;
-            before += hist[w * E + tid];
-            hist[w * E + tid] = 0;
-        }
-    }
-    __syncthreads();
-    place_pairs(a.ids, a.ids_dst, E, lo, hi, lane, hist + wave * E, base + wave * E);
-}
-
-// One block.  Stable counting sort of pairs by expert: per-wave histograms over contiguous pair
-// ranges give every (expert, wave) its own destination run, and inside a wave lanes holding the
-// same expert rank themselves by ballot, so compact slots keep ascending pair order.
-__global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
-    extern __shared__ int lds[];
-    if (blockIdx.x > 0 && a.tiles.src != nullptr) {
-        // blocks behind the first copy the activations into the pair layouts of the tile kernel while the first builds the plan
-        const int64_t item = static_cast<int64_t>(blockIdx.x - 1) * kPlanThreads + threadIdx.x;
-        tile_pack_item(item, a.tiles.src, a.tiles.dtype, a.tiles.rows, a.tiles.width, a.tiles.layouts, a.tiles.dst, a.tiles.layout_stride);
-        return;
-    }
-    if (blockIdx.x > 0) {
-        // blocks behind the first pack one activation row each while the first builds the plan
-        const int row = blockIdx.x - 1;
-        const int element = a.pack.dtype == MFQ_AMD_F32 ? 4 : 2;
-        xpack_row(static_cast<const char*>(a.pack.src) + static_cast<int64_t>(row) * a.pack.width * element, a.pack.dtype,
-                  a.pack.vector_ok != 0, a.pack.width, a.pack.dst + row * a.pack.stride, reinterpret_cast<float*>(lds));
-        return;
-    }
-    const int E = a.experts;
-    constexpr int kWaves = kPlanThreads / 64;
-    int* hist = lds;                    // [kWaves][E]
-    int* cnt = hist + kWaves * E;       // [E]
-    int* start = cnt + E;               // [E]
-    int* scratch = start + E;           // [kWaves]
-    int* wave_items = scratch + kWaves; // [K_CLASS_COUNT][kWaves]
-    int* wave_tiles = wave_items + K_CLASS_COUNT * kWaves;
-    int* totals = wave_tiles + K_CLASS_COUNT * kWaves;   // distinct, pad, 64-bit byte total
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-    for (int i = tid; i < kWaves * E; i += kPlanThreads) hist[i] = 0;
-    lds_barrier();
-    int lo, hi;
-    wave_range(a.pairs, kWaves, wave, 0, lo, hi);
-    count_ids(a.ids, E, lo, hi, lane, hist + wave * E);
-    lds_barrier();
-    int count = 0;
-    if (tid < E) {
-        for (int w = 0; w < kWaves; ++w) { const int c = hist[w * E + tid]; hist[w * E + tid] = count; count += c; }
-        cnt[tid] = count;
-        a.counts[tid] = count;
-    }
-    const int pair_scan = block_inclusive_scan(tid < E ? count : 0, scratch);
-    const int route_tiles = tid < E ? (count + a.tile_m - 1) / a.tile_m : 0;
-    const int tile_scan = block_inclusive_scan(route_tiles, scratch);
-    const bool want_route_tiles = a.tile_bounds != nullptr && a.tile_experts != nullptr;
-    if (tid < E) {
-        start[tid] = pair_scan - count;
-        a.expert_bounds[tid + 1] = pair_scan;
-        if (want_route_tiles) {
-            a.tile_bounds[tid + 1] = tile_scan;
-            for (int t = tile_scan - route_tiles; t < tile_scan; ++t) a.tile_experts[t] = tid;
-        }
-    }
-    if (tid == 0) { a.expert_bounds[0] = 0; if (want_route_tiles) a.tile_bounds[0] = 0; }
-    lds_barrier();
-
-    if (a.wave_base != nullptr) {
-        // the pairs are placed by route_scatter_kernel, one block per wave range of this kernel
-        if (tid < E)
-            for (int w = 0; w < kWaves; ++w) a.wave_base[w * E + tid] = start[tid] + hist[w * E + tid];
-    } else {
-        place_pairs(a.ids, a.ids_dst, E, lo, hi, lane, hist + wave * E, start);
-    }
-
     const PlanExtras& x = a.extras;
-    if (x.items == nullptr) return;
     // Work lists per slot: active experts ordered by (kernel class, expert id), and their prefill
     // tiles in the same order.  Ranks come from per-class ballots inside a wave plus a small table
     // of per-(class, wave) totals.
@@ -704,6 +618,118 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
     }
     __syncthreads();
     if (tid == 0) { *x.touched_bytes = static_cast<int64_t>(*total_bytes); *x.distinct = *total_distinct; }
+}
+
+// Second kernel of a large plan: block b places the pairs of wave range b of route_plan_kernel, split
+// again over its own waves; wave_base[b][e] (written by route_plan_kernel) is where the block's run of
+// expert e starts.
+__global__ void __launch_bounds__(kPlanThreads) route_scatter_kernel(PlanArgs a) {
+    extern __shared__ int lds[];
+    const int E = a.experts;
+    constexpr int kWaves = kPlanThreads / 64;
+    int* hist = lds;                    // [kWaves][E]: counts, then pairs placed so far
+    int* base = hist + kWaves * E;      // [kWaves][E]: start of the run of (wave, expert)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (blockIdx.x == kWaves) {
+        // the block behind the placing ones: the work lists, from the counts and bounds route_plan_kernel left
+        int* cnt = lds;
+        int* start = cnt + E;
+        int* scratch = start + E;
+        int* wave_items = scratch + kWaves;
+        int* wave_tiles = wave_items + K_CLASS_COUNT * kWaves;
+        int* totals = wave_tiles + K_CLASS_COUNT * kWaves;
+        if (tid < E) { cnt[tid] = a.counts[tid]; start[tid] = a.expert_bounds[tid]; }
+        plan_work_lists(a, lds, cnt, start, scratch, wave_items, wave_tiles, totals);
+        return;
+    }
+    int block_lo, block_hi, lo, hi;
+    wave_range(a.pairs, kWaves, blockIdx.x, 0, block_lo, block_hi);
+    wave_range(block_hi - block_lo, kWaves, wave, block_lo, lo, hi);
+    for (int i = tid; i < kWaves * E; i += kPlanThreads) hist[i] = 0;
+    __syncthreads();
+    count_ids(a.ids, E, lo, hi, lane, hist + wave * E);
+    __syncthreads();
+    if (tid < E) {
+        int before = a.wave_base[blockIdx.x * E + tid];
+        for (int w = 0; w < kWaves; ++w) {
+            base[w * E + tid] = before;
+            before += hist[w * E + tid];
+            hist[w * E + tid] = 0;
+        }
+    }
+    __syncthreads();
+    place_pairs(a.ids, a.ids_dst, E, lo, hi, lane, hist + wave * E, base + wave * E);
+}
+
+// One block.  Stable counting sort of pairs by expert: per-wave histograms over contiguous pair
+// ranges give every (expert, wave) its own destination run, and inside a wave lanes holding the
+// same expert rank themselves by ballot, so compact slots keep ascending pair order.
+__global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
+    extern __shared__ int lds[];
+    if (blockIdx.x > 0 && a.tiles.src != nullptr) {
+        // blocks behind the first copy the activations into the pair layouts of the tile kernel while the first builds the plan
+        const int64_t item = static_cast<int64_t>(blockIdx.x - 1) * kPlanThreads + threadIdx.x;
+        tile_pack_item(item, a.tiles.src, a.tiles.dtype, a.tiles.rows, a.tiles.width, a.tiles.layouts, a.tiles.dst, a.tiles.layout_stride);
+        return;
+    }
+    if (blockIdx.x > 0) {
+        // blocks behind the first pack one activation row each while the first builds the plan
+        const int row = blockIdx.x - 1;
+        const int element = a.pack.dtype == MFQ_AMD_F32 ? 4 : 2;
+        xpack_row(static_cast<const char*>(a.pack.src) + static_cast<int64_t>(row) * a.pack.width * element, a.pack.dtype,
+                  a.pack.vector_ok != 0, a.pack.width, a.pack.dst + row * a.pack.stride, reinterpret_cast<float*>(lds));
+        return;
+    }
+    const int E = a.experts;
+    constexpr int kWaves = kPlanThreads / 64;
+    int* hist = lds;                    // [kWaves][E]
+    int* cnt = hist + kWaves * E;       // [E]
+    int* start = cnt + E;               // [E]
+    int* scratch = start + E;           // [kWaves]
+    int* wave_items = scratch + kWaves; // [K_CLASS_COUNT][kWaves]
+    int* wave_tiles = wave_items + K_CLASS_COUNT * kWaves;
+    int* totals = wave_tiles + K_CLASS_COUNT * kWaves;   // distinct, pad, 64-bit byte total
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    for (int i = tid; i < kWaves * E; i += kPlanThreads) hist[i] = 0;
+    lds_barrier();
+    int lo, hi;
+    wave_range(a.pairs, kWaves, wave, 0, lo, hi);
+    count_ids(a.ids, E, lo, hi, lane, hist + wave * E);
+    lds_barrier();
+    int count = 0;
+    if (tid < E) {
+        for (int w = 0; w < kWaves; ++w) { const int c = hist[w * E + tid]; hist[w * E + tid] = count; count += c; }
+        cnt[tid] = count;
+        a.counts[tid] = count;
+    }
+    const int pair_scan = block_inclusive_scan(tid < E ? count : 0, scratch);
+    const int route_tiles = tid < E ? (count + a.tile_m - 1) / a.tile_m : 0;
+    const int tile_scan = block_inclusive_scan(route_tiles, scratch);
+    const bool want_route_tiles = a.tile_bounds != nullptr && a.tile_experts != nullptr;
+    if (tid < E) {
+        start[tid] = pair_scan - count;
+        a.expert_bounds[tid + 1] = pair_scan;
+        if (want_route_tiles) {
+            a.tile_bounds[tid + 1] = tile_scan;
+            for (int t = tile_scan - route_tiles; t < tile_scan; ++t) a.tile_experts[t] = tid;
+        }
+    }
+    if (tid == 0) { a.expert_bounds[0] = 0; if (want_route_tiles) a.tile_bounds[0] = 0; }
+    lds_barrier();
+
+    if (a.wave_base != nullptr) {
+        // the pairs are placed by route_scatter_kernel, one block per wave range of this kernel
+        if (tid < E)
+            for (int w = 0; w < kWaves; ++w) a.wave_base[w * E + tid] = start[tid] + hist[w * E + tid];
+    } else {
+        place_pairs(a.ids, a.ids_dst, E, lo, hi, lane, hist + wave * E, start);
+    }
+
+    const PlanExtras& x = a.extras;
+    if (x.items == nullptr) return;
+    if (a.wave_base != nullptr && a.lists_in_scatter) return;      // the block behind route_scatter_kernel's builds them meanwhile
+    plan_work_lists(a, lds, cnt, start, scratch, wave_items, wave_tiles, totals);
 }
 
 // The same plan for at most kPlanThreads pairs (decode): one thread per pair and per expert, no
@@ -1204,12 +1230,18 @@ void launch_route_plan(const PlanArgs& args, hipStream_t stream) {
         const int64_t items = static_cast<int64_t>(args.tiles.rows) * (args.tiles.width / dev::kLaneColumns);
         spare_blocks = static_cast<int>((items + kPlanThreads - 1) / kPlanThreads);
     }
-    hipLaunchKernelGGL(dev::route_plan_kernel, dim3(1 + spare_blocks), dim3(kPlanThreads), lds, stream, args);
+    // with a scatter launch behind it, the plan kernel stops after the bounds; the work lists are built by one more
+    // block of the scatter launch, beside the blocks that place the pairs
+    PlanArgs large_args = args;
+    large_args.lists_in_scatter = args.wave_base != nullptr && args.extras.items != nullptr ? 1 : 0;
+    hipLaunchKernelGGL(dev::route_plan_kernel, dim3(1 + spare_blocks), dim3(kPlanThreads), lds, stream, large_args);
     check_launch("route_plan_kernel");
     if (args.wave_base != nullptr) {
-        const size_t scatter_lds = sizeof(int) * 2 * (kPlanThreads / 64) * args.experts;
+        const size_t place_lds = sizeof(int) * 2 * (kPlanThreads / 64) * args.experts;
+        const size_t scatter_lds = place_lds > lds ? place_lds : lds;       // the lists block lays its LDS out as the plan kernel does
         if (scatter_lds > 64 * 1024) (void)device_state();
-        hipLaunchKernelGGL(dev::route_scatter_kernel, dim3(kPlanThreads / 64), dim3(kPlanThreads), scatter_lds, stream, args);
+        hipLaunchKernelGGL(dev::route_scatter_kernel, dim3(kPlanThreads / 64 + large_args.lists_in_scatter), dim3(kPlanThreads), scatter_lds,
+                           stream, large_args);
         check_launch("route_scatter_kernel");
     }
 }

@@ -130,6 +130,7 @@ struct PlanArgs {
     PlanExtras extras;        // extras.items == nullptr: plain route plan
     PlanPack pack;
     PlanTilePack tiles;
+    int32_t lists_in_scatter;   // large plans (set by the launcher): the work lists are built by a block of the scatter launch
     PlanRoute route;
 };
 
