@@ -179,15 +179,25 @@ struct TopkScratch {
 // group falls back to one selection round per rank: the best of the lane candidates by lane exchanges, and the
 // winning lane rescans its entries.  Both give the same ids.
 //
-// Every thread of the block calls it (block-wide barriers inside); groups with active == false select nothing.
+// Every lane of a token's wave calls it (the lanes of a wave synchronise among themselves, no block barrier); groups with
+// active == false select nothing.  A caller that reads `local_ids` from other waves puts its own barrier in between.
 // `local_ids`, when given, also receives the ids (any address space, e.g. LDS).
+// The lanes of a token (half a wave or a whole one) exchange data through LDS: the LDS operations of a wave complete
+// in program order, so it is enough that the wave waits for its own and the compiler keeps the order.  A block barrier
+// here would make every wave of the block wait for every other token's, and for the acknowledgement of its own global
+// stores each time.
+__device__ __forceinline__ void wave_lds_sync() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+}
+
 template <int SLOTS, int LANES = 32>
 __device__ __forceinline__ void topk_token(const void* logits, int dtype, int token, bool active, int experts, int top_k,
                                            int normalize, float norm_floor, float scale, int32_t* ids,
                                            float* weights, int* local_ids, TopkScratch* scratch) {
     static_assert(LANES == 32 || LANES == 64, "a token takes half a wave or a whole one");
     const int lane = threadIdx.x & (LANES - 1);
-    const bool busy = __ballot(active) != 0ull;          // waves without a token only keep the barriers
+    const bool busy = __ballot(active) != 0ull;          // waves without a token have nothing to do
     float cached[SLOTS];
     float total = 1.0f;
     int lane_best = -1;
@@ -255,7 +265,7 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
         scratch->lane_best[lane] = lane_best;
         if (lane == 0) { scratch->threshold = 0x7fffffff; scratch->count = 0; }
     }
-    __syncthreads();
+    wave_lds_sync();
     if (busy) {
         // the top_k-th largest lane maximum: the smallest one that fewer than top_k others exceed
         int greater = 0;
@@ -266,7 +276,7 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
         }
         if (greater < top_k) atomicMin(&scratch->threshold, lane_best);
     }
-    __syncthreads();
+    wave_lds_sync();
     if (busy) {
         const int bound = scratch->threshold - 8 > 0 ? scratch->threshold - 8 : 0;
         int mine = 0;
@@ -283,7 +293,7 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
             }
         }
     }
-    __syncthreads();
+    wave_lds_sync();
     const int found = busy ? scratch->count : 0;
     // (numerators below 2^-100 can give subnormal probabilities, where many more numerators share one quotient)
     const bool by_rounds = active && (found > kTopkCandidates || found < top_k || scratch->threshold < 0x0D800000);
@@ -301,13 +311,13 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
             }
         }
     }
-    __syncthreads();
+    wave_lds_sync();
     if (busy && active && !by_rounds) {
 #pragma unroll
         for (int j = 0; j < kTopkCandidates / LANES; ++j)
             if (lane + LANES * j < found) scratch->candidates[lane + LANES * j] = mine2[j];
     }
-    __syncthreads();
+    wave_lds_sync();
     if (busy && active && !by_rounds) {
 #pragma unroll
         for (int j = 0; j < kTopkCandidates / LANES; ++j) {
@@ -362,7 +372,7 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
             }
         }
     }
-    __syncthreads();
+    wave_lds_sync();
     if (busy) {
         const float selected = active && lane < top_k ? __uint_as_float(static_cast<uint32_t>(scratch->selected[lane])) : 0.0f;
         float denominator = 1.0f;
