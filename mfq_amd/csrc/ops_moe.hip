@@ -116,11 +116,18 @@ __device__ __forceinline__ void hidden_to_lds(const RowsArgs& a, int pair, Hidde
     const uint16_t* gate = a.gu + static_cast<int64_t>(pair) * 2 * a.in_width;
     const uint16_t* up = gate + a.in_width;
     uint32_t largest = 0u;
-    for (int col = threadIdx.x; col < a.in_width; col += blockDim.x) {
-        const uint16_t h = swiglu_bits(gate[col], up[col], a.swiglu_limit, a.sigmoid);
-        hidden->values[col] = h;
+    auto count = [&](uint16_t h) {
         const uint32_t magnitude = h & 0x7fffu;
         largest = magnitude > largest && magnitude <= 0x7c00u ? magnitude : largest;     // NaN does not count, as with fmaxf
+    };
+    // two columns per thread (rows are multiples of 32 columns and start at multiples of four bytes): a row of 512 columns
+    // is one round of loads and one round of table lookups for the block
+    for (int col = 2 * threadIdx.x; col < a.in_width; col += 2 * blockDim.x) {
+        const uint32_t g = *reinterpret_cast<const uint32_t*>(gate + col), u = *reinterpret_cast<const uint32_t*>(up + col);
+        const uint16_t lo = swiglu_bits(static_cast<uint16_t>(g & 0xffffu), static_cast<uint16_t>(u & 0xffffu), a.swiglu_limit, a.sigmoid);
+        const uint16_t hi = swiglu_bits(static_cast<uint16_t>(g >> 16), static_cast<uint16_t>(u >> 16), a.swiglu_limit, a.sigmoid);
+        *reinterpret_cast<uint32_t*>(&hidden->values[col]) = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+        count(lo); count(hi);
     }
     largest = wave_max_u32(largest);       // the bits of non-negative halves order like their values
     if (threadIdx.x % kWave == 0) hidden->wave_largest[threadIdx.x / kWave] = largest;
@@ -243,11 +250,26 @@ __global__ void __launch_bounds__(256) swiglu_pack_kernel(const uint16_t* gate, 
     uint16_t* staged = reinterpret_cast<uint16_t*>(lds);
     float* scratch = reinterpret_cast<float*>(lds + ((static_cast<size_t>(inner) * 2 + 15) / 16) * 16);
     const int64_t row = blockIdx.x;
-    for (int col = threadIdx.x; col < inner; col += blockDim.x) {
-        const uint16_t gb = gate[row * gate_stride + col], ub = up[row * gate_stride + col];
-        const uint16_t result = swiglu_bits(gb, ub, limit, table);
-        hidden[row * inner + col] = result;
-        staged[col] = result;
+    const bool pairs_ok = inner % 2 == 0 && gate_stride % 2 == 0 && (reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up) |
+                                                                     reinterpret_cast<uintptr_t>(hidden)) % 4 == 0;
+    if (pairs_ok) {
+        // two columns per thread: a row of 512 columns is one round of loads and one round of table lookups for the block
+        // (one column per thread made it two of each, one after the other)
+        for (int col = 2 * threadIdx.x; col < inner; col += 2 * blockDim.x) {
+            const uint32_t g = *reinterpret_cast<const uint32_t*>(gate + row * gate_stride + col);
+            const uint32_t u = *reinterpret_cast<const uint32_t*>(up + row * gate_stride + col);
+            const uint32_t lo = swiglu_bits(static_cast<uint16_t>(g & 0xffffu), static_cast<uint16_t>(u & 0xffffu), limit, table);
+            const uint32_t hi = swiglu_bits(static_cast<uint16_t>(g >> 16), static_cast<uint16_t>(u >> 16), limit, table);
+            *reinterpret_cast<uint32_t*>(hidden + row * inner + col) = lo | (hi << 16);
+            *reinterpret_cast<uint32_t*>(staged + col) = lo | (hi << 16);
+        }
+    } else {
+        for (int col = threadIdx.x; col < inner; col += blockDim.x) {
+            const uint16_t gb = gate[row * gate_stride + col], ub = up[row * gate_stride + col];
+            const uint16_t result = swiglu_bits(gb, ub, limit, table);
+            hidden[row * inner + col] = result;
+            staged[col] = result;
+        }
     }
     __syncthreads();
     xpack_row(staged, MFQ_AMD_F16, true, inner, packed + row * packed_stride, scratch);
