@@ -256,15 +256,37 @@ __device__ __forceinline__ void nvq_fast_tables(const mfq_amd_projection& p, uns
     const int entries = nvq_format_entries(p.format);
     const int banks = jsc ? static_cast<uint8_t>(meta[1]) : 1;
     const uint8_t* tables = reinterpret_cast<const uint8_t*>(meta) + (jsc ? 64 : 0);
-    for (int i = threadIdx.x; i < banks * entries; i += blockDim.x) {
-        const uint32_t word = load_u32_unaligned(tables + 4 * i);
-        half2_t lo, hi;
-        lo[0] = static_cast<_Float16>(static_cast<float>(word & 0xffu));
-        lo[1] = static_cast<_Float16>(static_cast<float>((word >> 8) & 0xffu));
-        hi[0] = static_cast<_Float16>(static_cast<float>((word >> 16) & 0xffu));
-        hi[1] = static_cast<_Float16>(static_cast<float>(word >> 24));
-        book[2 * i] = __builtin_bit_cast(uint32_t, lo);
-        book[2 * i + 1] = __builtin_bit_cast(uint32_t, hi);
+    // Four entries (16 bytes of the pool's table) per thread and pass, and the loads of up to four passes requested
+    // before the first entry is converted: with one entry per pass a block of 256 threads made sixteen dependent
+    // round trips for a table of 4096 entries, more than the rows of a down block take to multiply.
+    constexpr int kPasses = 4;
+    const int total = banks * entries;                 // a multiple of four (256, 512 or 1024 entries per bank)
+    for (int first = 0; first < total; first += kPasses * 4 * static_cast<int>(blockDim.x)) {
+        u32x4 words[kPasses];
+#pragma unroll
+        for (int pass = 0; pass < kPasses; ++pass) {
+            const int i = first + 4 * (pass * static_cast<int>(blockDim.x) + static_cast<int>(threadIdx.x));
+            words[pass] = i < total ? *(const MFQ_GLOBAL u32x4_u*)(tables + 4 * i) : u32x4{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int pass = 0; pass < kPasses; ++pass) {
+            const int i = first + 4 * (pass * static_cast<int>(blockDim.x) + static_cast<int>(threadIdx.x));
+            if (i >= total) continue;
+            u32x4 out[2];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t word = words[pass][e];
+                half2_t lo, hi;
+                lo[0] = static_cast<_Float16>(static_cast<float>(word & 0xffu));
+                lo[1] = static_cast<_Float16>(static_cast<float>((word >> 8) & 0xffu));
+                hi[0] = static_cast<_Float16>(static_cast<float>((word >> 16) & 0xffu));
+                hi[1] = static_cast<_Float16>(static_cast<float>(word >> 24));
+                out[e / 2][2 * (e % 2)] = __builtin_bit_cast(uint32_t, lo);
+                out[e / 2][2 * (e % 2) + 1] = __builtin_bit_cast(uint32_t, hi);
+            }
+            *reinterpret_cast<u32x4*>(book + 2 * i) = out[0];
+            *reinterpret_cast<u32x4*>(book + 2 * i + 4) = out[1];
+        }
     }
     if (threadIdx.x < 128) {
         const uint32_t mask7 = threadIdx.x;
