@@ -165,15 +165,19 @@ __global__ void __launch_bounds__(256) gemv_fast_kernel(mfq_amd_projection p, in
                                                         int x_dtype, int batch, int64_t x_stride, float* y,
                                                         int64_t y_stride, int vector_ok) {
     extern __shared__ unsigned char lds[];
-    if (FastClass<CLS>::kNvq) {
-        nvq_fast_tables(p, lds);
-        __syncthreads();
-    }
+    // the LDS tables of an NVQ pool are built behind the first requests for packed rows (every wave of the block
+    // takes part: there is a barrier inside)
+    auto prologue = [&] {
+        if (FastClass<CLS>::kNvq) {
+            nvq_fast_tables(p, lds);
+            __syncthreads();
+        }
+    };
     const FastCtx<CLS> ctx = fast_ctx<CLS>(p, local_expert, lds);
     constexpr int kRowsPerWave = SLOTS * (kWave / LPR);
     const int wave = uniform(static_cast<int>(threadIdx.x / kWave));
     const int row_begin = (blockIdx.x * 4 + wave) * kRowsPerWave;
-    if (row_begin >= p.output_rows) return;
+    if (row_begin >= p.output_rows) { prologue(); return; }
     const int row_end = row_begin + kRowsPerWave < p.output_rows ? row_begin + kRowsPerWave : p.output_rows;
     const int element = x_dtype == MFQ_AMD_F32 ? 4 : 2;
     constexpr int kRing = SLABS > 1 ? 4 : (FastClass<CLS>::kRing < SLOTS ? FastClass<CLS>::kRing : SLOTS);
@@ -185,7 +189,7 @@ __global__ void __launch_bounds__(256) gemv_fast_kernel(mfq_amd_projection p, in
         xs[n] = XSource{static_cast<const char*>(x) + static_cast<int64_t>(token) * x_stride * element, x_dtype, vector_ok != 0, nullptr};
     }
     fast_rows<CLS, LPR, SLABS, NT, kRing, kXRaw, SLOTS>(ctx, xs, p.input_width, row_begin, row_end, p.output_rows,
-        [&](int n, int row, float value) { if (first + n < batch) y[static_cast<int64_t>(first + n) * y_stride + row] = value; });
+        [&](int n, int row, float value) { if (first + n < batch) y[static_cast<int64_t>(first + n) * y_stride + row] = value; }, prologue);
 }
 
 struct GemvFastLaunch {
