@@ -83,7 +83,23 @@ template <int CTRL>
 __device__ __forceinline__ float dpp(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
 }
-__device__ __forceinline__ float lane_xor(float v, int mask) { return __shfl_xor(v, mask, kWave); }
+// The lane's value and that of the lane DISTANCE (16 or 32) positions away, in an order that depends on the lane: for
+// operations that commute.  One register swap between the rows of the wave, where a shuffle is an LDS round trip.
+template <int DISTANCE>
+__device__ __forceinline__ void lane_and_partner(float v, float& one, float& other) {
+    static_assert(DISTANCE == 16 || DISTANCE == 32, "rows of 16 lanes or halves of 32");
+    const unsigned bits = __builtin_bit_cast(unsigned, v);
+    const auto swapped = DISTANCE == 16 ? __builtin_amdgcn_permlane16_swap(bits, bits, false, false)
+                                        : __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    one = __builtin_bit_cast(float, static_cast<unsigned>(swapped[0]));
+    other = __builtin_bit_cast(float, static_cast<unsigned>(swapped[1]));
+}
+template <int DISTANCE>
+__device__ __forceinline__ float add_partner(float v) {
+    float one, other;
+    lane_and_partner<DISTANCE>(v, one, other);
+    return one + other;
+}
 
 // Every lane returns the maximum over the wave.
 __device__ __forceinline__ float wave_max(float v) {
@@ -91,9 +107,11 @@ __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, dpp<0x4E>(v));
     v = fmaxf(v, dpp<0x141>(v));
     v = fmaxf(v, dpp<0x140>(v));
-    v = fmaxf(v, lane_xor(v, 16));
-    v = fmaxf(v, lane_xor(v, 32));
-    return v;
+    float one, other;
+    lane_and_partner<16>(v, one, other);
+    v = fmaxf(one, other);
+    lane_and_partner<32>(v, one, other);
+    return fmaxf(one, other);
 }
 
 // Sums N per-lane values over the LANES lanes of a row group in a fixed order.  On return the lane
@@ -132,8 +150,8 @@ __device__ __forceinline__ float reduce_values(const float (&v)[N], int lane) {
     a = a + dpp<0x124>(a);   // row_ror:4
     a = a + dpp<0x128>(a);   // row_ror:8
     if (LANES == 64) {
-        a = a + lane_xor(a, 16);
-        a = a + lane_xor(a, 32);
+        a = add_partner<16>(a);
+        a = add_partner<32>(a);
     }
     return a;
 }
@@ -421,6 +439,13 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t b
     return d;
 }
 
+// (a & mask) | (b & ~mask) in one instruction.
+__device__ __forceinline__ uint32_t bit_select(uint32_t mask, uint32_t a, uint32_t b) {
+    uint32_t d;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(d) : "s"(mask), "v"(a), "v"(b));
+    return d;
+}
+
 // fp16 bit pattern of 2^LOG2, in both halves.  A template constant, not a function of a float: a loop over
 // floats is not folded by the compiler, and as a call it ran (ten iterations per use) inside the tile kernel's steps.
 template <int LOG2>
@@ -469,7 +494,9 @@ __device__ __forceinline__ void chunk_pairs(const FastRaw<CLS>& raw, int j, uint
                          : j == 1 ? __builtin_amdgcn_alignbit(raw.q[1], raw.q[0], 24)
                          : j == 2 ? __builtin_amdgcn_alignbit(raw.q[2], raw.q[1], 16)
                                   : raw.q[2] >> 8;
-        const uint32_t u = ((w << 4) & 0xffff0000u) | (w & 0x0000ffffu);
+        // (one bit-select; left to the compiler the two halves are masked separately and every field below is then
+        // formed from both parts: two more instructions per chunk)
+        const uint32_t u = bit_select(0xffff0000u, w << 4, w);
         if constexpr (kDenormal) {
             t[0] = u & 0x00070007u; t[1] = u & 0x00380038u; t[2] = u & 0x01c001c0u; t[3] = (u >> 3) & 0x01c001c0u;
         } else {

@@ -15,6 +15,29 @@ __device__ __forceinline__ float uniform_lane(float v, int index) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), index));
 }
 
+// Value of lane `index` (0..15, a constant once the caller's loop is unrolled) of the lane's own row of 16 lanes:
+// one data-parallel move where a shuffle is an LDS round trip.
+__device__ __forceinline__ float row_lane(float v, int index) {
+    switch (index) {
+        case 0: return dpp<0x150>(v);   // row_newbcast:0
+        case 1: return dpp<0x151>(v);
+        case 2: return dpp<0x152>(v);
+        case 3: return dpp<0x153>(v);
+        case 4: return dpp<0x154>(v);
+        case 5: return dpp<0x155>(v);
+        case 6: return dpp<0x156>(v);
+        case 7: return dpp<0x157>(v);
+        case 8: return dpp<0x158>(v);
+        case 9: return dpp<0x159>(v);
+        case 10: return dpp<0x15A>(v);
+        case 11: return dpp<0x15B>(v);
+        case 12: return dpp<0x15C>(v);
+        case 13: return dpp<0x15D>(v);
+        case 14: return dpp<0x15E>(v);
+        default: return dpp<0x15F>(v);
+    }
+}
+
 // ------------------------------------------------------------ the row loop ----
 // Where one token's activations come from.
 struct XSource {
@@ -101,12 +124,14 @@ __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (
         return out;
     };
 
-    // Row scalars (NINT scale and minimum, NVQ anchor) of one pass over the ring: lane l holds those of
-    // the l-th row of the pass, one load per array and pass instead of one per row.
+    // Row scalars (NINT scale and minimum, NVQ anchor) of one pass over the ring, one load per array and pass instead
+    // of one per row.  64 lanes per row: lane l holds those of the l-th row of the pass.  16 lanes per row: lane i of
+    // a row of 16 lanes holds those of that lane group's row in the i-th slot of the pass.
     constexpr int kScalars = C::kNint ? 2 : C::kNvq ? 1 : 0;
     static_assert(RING * SUBS <= kWave && SLOTS * SUBS <= kWave, "the rows of a pass must fit the lanes of a wave");
+    static_assert(SUBS == 1 || (LPR == 16 && RING <= 16 && SLOTS <= 16), "a slot of the pass per lane of a row of 16");
     auto fetch_scalars = [&](int slot, float (&values)[2]) {
-        int row = row_begin + slot * SUBS + lane;
+        int row = SUBS == 1 ? row_begin + slot + lane : row_begin + (slot + li) * SUBS + sub;
         row = row < out_rows ? row : out_rows - 1;
         values[0] = kScalars >= 1 ? gload<float>(c.f3 + row) : 0.0f;
         values[1] = kScalars >= 2 ? gload<float>(c.f4 + row) : 0.0f;
@@ -173,8 +198,8 @@ __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (
 #pragma unroll
                 for (int n = 0; n < NT; ++n) row_v[n] = 0.0f;
                 float rs = 0.0f, rm = 0.0f;
-                if (kScalars >= 1) rs = SUBS == 1 ? uniform_lane(scalars[0], k) : __shfl(scalars[0], k * SUBS + sub, kWave);
-                if (kScalars >= 2) rm = SUBS == 1 ? uniform_lane(scalars[1], k) : __shfl(scalars[1], k * SUBS + sub, kWave);
+                if (kScalars >= 1) rs = SUBS == 1 ? uniform_lane(scalars[0], k) : row_lane(scalars[0], k);
+                if (kScalars >= 2) rm = SUBS == 1 ? uniform_lane(scalars[1], k) : row_lane(scalars[1], k);
 #pragma unroll
                 for (int s = 0; s < SLABS; ++s) {
                     if (s == 0 && !C::kNvq) fast_accumulate<CLS, NT, IB, false>(c, blocks[s], with_levels(ring[d][s]), rs, rm, x[s], row_v);
@@ -214,11 +239,11 @@ __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (
                 float row_v[NT];
 #pragma unroll
                 for (int n = 0; n < NT; ++n) row_v[n] = 0.0f;
-                // the scalars of the slot's row: lane d of the pass for 64 lanes per row, else the lane that
-                // matches this lane's row
+                // the scalars of the slot's row: lane d of the pass for 64 lanes per row, else lane d of the lane's
+                // own row of 16
                 float rs = 0.0f, rm = 0.0f;
-                if (kScalars >= 1) rs = SUBS == 1 ? uniform_lane(scalars[0], d) : __shfl(scalars[0], d * SUBS + sub, kWave);
-                if (kScalars >= 2) rm = SUBS == 1 ? uniform_lane(scalars[1], d) : __shfl(scalars[1], d * SUBS + sub, kWave);
+                if (kScalars >= 1) rs = SUBS == 1 ? uniform_lane(scalars[0], d) : row_lane(scalars[0], d);
+                if (kScalars >= 2) rm = SUBS == 1 ? uniform_lane(scalars[1], d) : row_lane(scalars[1], d);
 #pragma unroll
                 for (int s = 0; s < SLABS; ++s) {
                     if (s == 0 && !C::kNvq) fast_accumulate<CLS, NT, IB, false>(c, blocks[s], with_levels(ring[d][s]), rs, rm, x[s], row_v);
