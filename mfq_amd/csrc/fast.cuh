@@ -679,7 +679,8 @@ __device__ __forceinline__ void fast_accumulate(const FastCtx<CLS>& c, const Lan
                         if (j < 3) after[j][n] = run[n];
                     }
                 }
-                const bool from1 = (b.sel & 2u) != 0, from2 = (b.sel & 4u) != 0, from3 = (b.sel & 8u) != 0;
+                // (groups of 24 columns: the last chunk always lies in the second group)
+                const bool from1 = (b.sel & 2u) != 0, from2 = (b.sel & 4u) != 0, from3 = C::kGs == 24 || (b.sel & 8u) != 0;
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
                     const float first = from1 ? after[0][n] : from2 ? after[1][n] : from3 ? after[2][n] : run[n];
@@ -746,9 +747,11 @@ struct WeightBlock {
 
 // `scales`, `minima`: NINT: the levels of the block's first group in bits 0..7 and of the next group in bits 8..15;
 // NVQ: the block's four sign masks from bit 0, and the states of its two groups from bit 0.
+// `live` = false: every weight of the block comes out as zero (a lane block behind the end of the row, whose packed data
+// is that of a valid block): the factors are zeroed here, once per block, so the chunks need no test.
 template <int CLS>
 __device__ __forceinline__ WeightBlock<CLS> weight_block(const FastCtx<CLS>& c, const LaneBlock& b, const FastRaw<CLS>& raw,
-                                                         const WeightRow<CLS>& r, uint32_t scales, uint32_t minima) {
+                                                         const WeightRow<CLS>& r, uint32_t scales, uint32_t minima, bool live = true) {
     using C = FastClass<CLS>;
     WeightBlock<CLS> k{};
     k.sel = b.sel;
@@ -757,16 +760,17 @@ __device__ __forceinline__ WeightBlock<CLS> weight_block(const FastCtx<CLS>& c, 
         k.masks = scales;
         k.q2 = raw.q[2] >> (raw.b & 0xffu);
         const uint32_t state0 = states & 15u, state1 = (states >> 4) & 15u;
-        k.scale[0] = splat_half(c.multiplier[state0]);
-        k.scale[1] = splat_half(c.multiplier[state1]);
+        k.scale[0] = splat_half(live ? c.multiplier[state0] : 0.0f);
+        k.scale[1] = splat_half(live ? c.multiplier[state1] : 0.0f);
         typedef const __attribute__((address_space(3))) unsigned char* lds_bytes;
         k.bank_at[0] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_bytes)(c.codebook + c.bank_byte[state0])));
         k.bank_at[1] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_bytes)(c.codebook + c.bank_byte[state1])));
         k.signs_at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_bytes)c.signs));
     } else if constexpr (C::kMx) {
-        k.block_scale = bits_to_float(raw.a ? (raw.a << 23) : 0x00400000u);
+        k.block_scale = live ? bits_to_float(raw.a ? (raw.a << 23) : 0x00400000u) : 0.0f;
     } else {
         constexpr float center = static_cast<float>(1 << (C::kBits - 1));
+        if (!live) { scales = 0u; minima = 0u; }   // levels of zero: s (q - c) + (s c - ratio m) = 0
         const float s0 = r.coef * static_cast<float>(scales & 0xffu), s1 = r.coef * static_cast<float>((scales >> 8) & 0xffu);
         const float m0 = static_cast<float>(minima & 0xffu), m1 = static_cast<float>((minima >> 8) & 0xffu);
         k.level[0] = splat_half(s0);
@@ -822,8 +826,10 @@ __device__ __forceinline__ void chunk_weights(const WeightBlock<CLS>& k, const F
         } else {
             chunk_pairs<CLS, true>(raw, j, t);
         }
-        // dword j / 2 of a 2-bit block is one group; elsewhere sel flags the chunks of the second group
-        const bool second = C::kGs == 32 ? false : C::kBits == 2 ? j >= 2 : ((k.sel >> j) & 1u) != 0;
+        // dword j / 2 of a 2-bit block is one group; elsewhere sel flags the chunks of the second group (groups of 24
+        // columns: the first chunk of a block always lies in its first group and the last in its second)
+        const bool second = C::kGs == 32 ? false : C::kBits == 2 ? j >= 2
+                          : (C::kGs == 24 && j == 0) ? false : (C::kGs == 24 && j == 3) ? true : ((k.sel >> j) & 1u) != 0;
         const half2_t level = second ? k.level[1] : k.level[0], shift = second ? k.shift[1] : k.shift[0];
 #pragma unroll
         for (int m = 0; m < 4; ++m) {

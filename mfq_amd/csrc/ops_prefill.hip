@@ -442,21 +442,16 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
             uint32_t scales = 0, minima = 0;
             if constexpr (C::kNint) { scales = level_pair(0, t, b); minima = level_pair(1, t, b); }
             if constexpr (C::kNvq) side_pair(t, b, scales, minima);
-            block[t] = weight_block<CLS>(ctx, b, raw[t], scale[t], scales, minima);
+            // direct loads cannot blank the activations of lane blocks behind the end of the row (the converting path
+            // stores zeros there): their weights are made zero instead
+            block[t] = weight_block<CLS>(ctx, b, raw[t], scale[t], scales, minima, !(PACKED && ragged) || b.valid);
         }
         const unsigned char* x_tile = x_lds + (step & 1) * kFastXBytes + (PACKED ? 0 : n * kFastXRow + h * 64);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             uint32_t w[2][4];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                chunk_weights<CLS, IB>(block[t], raw[t], j, w[t]);
-                if (PACKED && ragged) {
-                    // direct loads cannot blank the lane blocks behind the end of the row: blank their weights
-#pragma unroll
-                    for (int m = 0; m < 4; ++m) w[t][m] = b.valid ? w[t][m] : 0u;
-                }
-            }
+            for (int t = 0; t < 2; ++t) chunk_weights<CLS, IB>(block[t], raw[t], j, w[t]);
             if (PACKED && j == 0) {
                 // The weights of this step have arrived (chunk 0 waited for them); the activations of the next
                 // step are requested now, so that no wait for older loads also waits for these.
