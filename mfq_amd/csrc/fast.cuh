@@ -747,11 +747,9 @@ struct WeightBlock {
 
 // `scales`, `minima`: NINT: the levels of the block's first group in bits 0..7 and of the next group in bits 8..15;
 // NVQ: the block's four sign masks from bit 0, and the states of its two groups from bit 0.
-// `live` = false: every weight of the block comes out as zero (a lane block behind the end of the row, whose packed data
-// is that of a valid block): the factors are zeroed here, once per block, so the chunks need no test.
 template <int CLS>
 __device__ __forceinline__ WeightBlock<CLS> weight_block(const FastCtx<CLS>& c, const LaneBlock& b, const FastRaw<CLS>& raw,
-                                                         const WeightRow<CLS>& r, uint32_t scales, uint32_t minima, bool live = true) {
+                                                         const WeightRow<CLS>& r, uint32_t scales, uint32_t minima) {
     using C = FastClass<CLS>;
     WeightBlock<CLS> k{};
     k.sel = b.sel;
@@ -760,17 +758,16 @@ __device__ __forceinline__ WeightBlock<CLS> weight_block(const FastCtx<CLS>& c, 
         k.masks = scales;
         k.q2 = raw.q[2] >> (raw.b & 0xffu);
         const uint32_t state0 = states & 15u, state1 = (states >> 4) & 15u;
-        k.scale[0] = splat_half(live ? c.multiplier[state0] : 0.0f);
-        k.scale[1] = splat_half(live ? c.multiplier[state1] : 0.0f);
+        k.scale[0] = splat_half(c.multiplier[state0]);
+        k.scale[1] = splat_half(c.multiplier[state1]);
         typedef const __attribute__((address_space(3))) unsigned char* lds_bytes;
         k.bank_at[0] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_bytes)(c.codebook + c.bank_byte[state0])));
         k.bank_at[1] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_bytes)(c.codebook + c.bank_byte[state1])));
         k.signs_at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_bytes)c.signs));
     } else if constexpr (C::kMx) {
-        k.block_scale = live ? bits_to_float(raw.a ? (raw.a << 23) : 0x00400000u) : 0.0f;
+        k.block_scale = bits_to_float(raw.a ? (raw.a << 23) : 0x00400000u);
     } else {
         constexpr float center = static_cast<float>(1 << (C::kBits - 1));
-        if (!live) { scales = 0u; minima = 0u; }   // levels of zero: s (q - c) + (s c - ratio m) = 0
         const float s0 = r.coef * static_cast<float>(scales & 0xffu), s1 = r.coef * static_cast<float>((scales >> 8) & 0xffu);
         const float m0 = static_cast<float>(minima & 0xffu), m1 = static_cast<float>((minima >> 8) & 0xffu);
         k.level[0] = splat_half(s0);

@@ -68,6 +68,9 @@ void launch_rows_fast(const RowsArgs& args, int slots, bool nvq, hipStream_t str
 void launch_rows_prefill(const RowsArgs& args, int slots, const int* present, const int* max_tiles, hipStream_t stream);
 // True when the streaming MFMA tile kernel serves rows of this width, activation type and alignment.
 bool tiles_fast_geometry(int in_width, int in_dtype, int in_vector_ok);
+// Whether the tile kernel can take the rows as packed fp16 copies (RowsArgs::in_tiles): whole steps of 128 columns and
+// a copy of less than 4 GB.
+bool tiles_packed_geometry(int in_width, int64_t in_rows);
 // Streaming MFMA tile kernel, one launch for every class; max_tiles bounds the tiles of a slot.
 // Tiles of pools marked kPoolExactOnly are skipped.
 void launch_tiles_fast(const RowsArgs& args, int slots, int max_tiles, bool nvq, hipStream_t stream);

@@ -880,7 +880,8 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         // blocks of the plan kernel (the plan itself keeps one CU busy)
         const int x_element = f->config.x_dtype == MFQ_AMD_F32 ? 4 : 2;
         const bool x_vector_ok = reinterpret_cast<uintptr_t>(x_dev) % 16 == 0 && (static_cast<int64_t>(H) * x_element) % 16 == 0;
-        const bool x_tiles = !decode && f->d_x_tiles != nullptr && tiles_fast_geometry(H, f->config.x_dtype, x_vector_ok);
+        const bool x_tiles = !decode && f->d_x_tiles != nullptr && tiles_fast_geometry(H, f->config.x_dtype, x_vector_ok) &&
+                             tiles_packed_geometry(H, tokens);
         if (x_tiles) {
             plan.tiles.src = x_dev; plan.tiles.dst = f->d_x_tiles; plan.tiles.layout_stride = static_cast<int64_t>(tokens) * H;
             plan.tiles.rows = tokens; plan.tiles.width = H; plan.tiles.dtype = f->config.x_dtype; plan.tiles.layouts = f->x_tile_layouts;
@@ -976,7 +977,7 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         f->mark(2, stream);
 
         const bool hidden_tiles = !decode && f->config.launch_mode == 0 && f->d_expert_info != nullptr &&
-                                  tiles_fast_geometry(I, MFQ_AMD_F16, 1);
+                                  tiles_fast_geometry(I, MFQ_AMD_F16, 1) && tiles_packed_geometry(I, pairs);
         if (fuse_swiglu) {
             // no kernel of its own
         } else if (hidden_tiles) {

@@ -181,7 +181,7 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
     const int n = lane & 31, h = lane >> 5;
     const int width = a.in_width, blocks = width / kLaneColumns;
     const int steps = (blocks + 3) / 4 * 2;            // 64 columns per step, an even number of steps
-    const bool ragged = blocks % 4 != 0;               // some step meets lane blocks beyond the row
+    const bool ragged = !PACKED && blocks % 4 != 0;    // some step meets lane blocks beyond the row (never with packed activations)
     const bool half_in = a.in_dtype == MFQ_AMD_F16;
 
     // activation staging: thread -> (pair of the tile, one of the two lane blocks of a step)
@@ -214,59 +214,38 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
     };
     // packed activations: the block copies the 32 MT rows the MFMAs read per step, a wave 8 rows of every 32
     // with one direct load of 8 rows x 128 bytes; lane -> (row 32 i + 8 wave + lane / 8, position lane % 8
-    // of the row in LDS)
-    const unsigned char* packed_row[MT];
-    int packed_piece[MT];
-    // When no step meets a lane block behind the end of the row and the copy of the activations is below 4 GB, the
-    // copies take their address as a scalar base (layout + step) plus a 32-bit lane offset that never changes: no
-    // vector arithmetic per step.
+    // of the row in LDS).  The launch has checked that no step meets a lane block behind the end of the row and that
+    // the copy of the activations is below 4 GB (tiles_packed_geometry), so a copy takes its address as a scalar base
+    // (layout + step) plus a 32-bit lane offset that never changes: no vector arithmetic per step.
     const unsigned char* packed_base = nullptr;
     uint32_t packed_offset[MT];
-    bool packed_scalar = false;
     if constexpr (PACKED) {
         const uint16_t* base = a.in_tiles + tile_layout<CLS>() * a.in_tiles_layout_stride;
         packed_base = reinterpret_cast<const unsigned char*>(base);
-        const int64_t rows_in = a.in_per_pair ? a.pairs : (a.pairs + a.top_k - 1) / a.top_k;
-        packed_scalar = !ragged && rows_in * width * 2 < (int64_t(1) << 32);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const int r = 32 * i + 8 * wave + lane / 8;
             const int pair = r < count ? a.ids_dst[begin + r] : -1;
             const int64_t from = pair < 0 ? 0 : a.in_per_pair ? pair : pair / a.top_k;
-            packed_row[i] = reinterpret_cast<const unsigned char*>(base + from * width);
-            packed_piece[i] = (lane % 8) ^ tile_swizzle(r);
-            packed_offset[i] = static_cast<uint32_t>(from * width * 2 + packed_piece[i] * 16);
+            const int piece = (lane % 8) ^ tile_swizzle(r);
+            packed_offset[i] = static_cast<uint32_t>(from * width * 2 + piece * 16);
         }
     }
     auto x_direct = [&](int step) {
-        if (packed_scalar) {
-            // the same address in every lane; said so for the "s" operand below
-            const uintptr_t address = reinterpret_cast<uintptr_t>(packed_base + step * 128);
-            const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(address)));
-            const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(address >> 32)));
-            const unsigned char* from = reinterpret_cast<const unsigned char*>((static_cast<uintptr_t>(hi) << 32) | lo);
-#pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                unsigned char* to = x_lds + (step & 1) * kFastXBytes + (32 * i + 8 * wave) * 128;
-                const uint32_t lds_at = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
-                    reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)(to)))));
-                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                             :: "v"(packed_offset[i]), "s"(from), "s"(lds_at) : "memory", "m0");
-            }
-            return;
-        }
+        // the same address in every lane; said so for the "s" operand below
+        const uintptr_t address = reinterpret_cast<uintptr_t>(packed_base + step * 128);
+        const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(address)));
+        const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(address >> 32)));
+        const unsigned char* from = reinterpret_cast<const unsigned char*>((static_cast<uintptr_t>(hi) << 32) | lo);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-            int cb = 2 * step + packed_piece[i] / 4;
-            cb = cb < blocks ? cb : blocks - 1;
-            const unsigned char* from = packed_row[i] + cb * 64 + (packed_piece[i] % 4) * 16;
             unsigned char* to = x_lds + (step & 1) * kFastXBytes + (32 * i + 8 * wave) * 128;
             // written as assembly so that the compiler does not make every later LDS read wait for it; the
             // waits that cover these loads are the explicit ones before the barriers
             const uint32_t lds_at = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
                 reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)(to)))));
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                         :: "v"(from), "s"(lds_at) : "memory", "m0");
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :: "v"(packed_offset[i]), "s"(from), "s"(lds_at) : "memory", "m0");
         }
     };
     // byte offsets of the operand pieces a lane reads inside a group of 32 rows; the swizzle of row
@@ -442,9 +421,7 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
             uint32_t scales = 0, minima = 0;
             if constexpr (C::kNint) { scales = level_pair(0, t, b); minima = level_pair(1, t, b); }
             if constexpr (C::kNvq) side_pair(t, b, scales, minima);
-            // direct loads cannot blank the activations of lane blocks behind the end of the row (the converting path
-            // stores zeros there): their weights are made zero instead
-            block[t] = weight_block<CLS>(ctx, b, raw[t], scale[t], scales, minima, !(PACKED && ragged) || b.valid);
+            block[t] = weight_block<CLS>(ctx, b, raw[t], scale[t], scales, minima);
         }
         const unsigned char* x_tile = x_lds + (step & 1) * kFastXBytes + (PACKED ? 0 : n * kFastXRow + h * 64);
 #pragma unroll
@@ -865,6 +842,10 @@ void raise_prefill_limits() {
                                 hipFuncAttributeMaxDynamicSharedMemorySize, dev::kSigmoidTableBytes));
 }
 
+bool tiles_packed_geometry(int in_width, int64_t in_rows) {
+    return in_width % (4 * dev::kLaneColumns) == 0 && in_rows * in_width * 2 < (int64_t(1) << 32);
+}
+
 bool tiles_fast_geometry(int in_width, int in_dtype, int in_vector_ok) {
     return in_width % dev::kLaneColumns == 0 && in_width >= 2 * dev::kLaneColumns && in_dtype != MFQ_AMD_F32 && in_vector_ok != 0;
 }
@@ -879,6 +860,8 @@ void launch_tiles_fast(const RowsArgs& args, int slots, int max_tiles, bool nvq,
     (void)nvq;   // the table region also holds the NINT level windows
     const int bytes = dev::kTilesFastLdsBytes;   // more than the default 64 KB of dynamic LDS: raised by device_state()
     (void)device_state();
+    MFQ_REQUIRE(a.in_tiles == nullptr || tiles_packed_geometry(a.in_width, a.in_per_pair ? a.pairs : (a.pairs + a.top_k - 1) / a.top_k),
+                "packed activation tiles need rows of whole steps and a copy below 4 GB");
     if (a.in_tiles != nullptr) hipLaunchKernelGGL(dev::moe_tiles_fast_kernel<true>, grid, dim3(256), bytes, stream, a);
     else hipLaunchKernelGGL(dev::moe_tiles_fast_kernel<false>, grid, dim3(256), bytes, stream, a);
     check_launch("moe_tiles_fast_kernel");
