@@ -679,8 +679,7 @@ __device__ __forceinline__ void fast_accumulate(const FastCtx<CLS>& c, const Lan
                         if (j < 3) after[j][n] = run[n];
                     }
                 }
-                // (groups of 24 columns: the last chunk always lies in the second group)
-                const bool from1 = (b.sel & 2u) != 0, from2 = (b.sel & 4u) != 0, from3 = C::kGs == 24 || (b.sel & 8u) != 0;
+                const bool from1 = (b.sel & 2u) != 0, from2 = (b.sel & 4u) != 0, from3 = (b.sel & 8u) != 0;
 #pragma unroll
                 for (int n = 0; n < NT; ++n) {
                     const float first = from1 ? after[0][n] : from2 ? after[1][n] : from3 ? after[2][n] : run[n];
