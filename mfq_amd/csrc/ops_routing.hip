@@ -136,11 +136,52 @@ __device__ __forceinline__ float load_logit(const void* logits, int dtype, int64
     return raw != raw ? -3.402823466e+38f : raw;
 }
 
-// Lane 0 of a 32-lane shuffle-down tree, offsets 16, 8, 4, 2, 1.
+// Exchanges between lanes without the LDS round trip of a shuffle.  swap_rows<16>: the value of the lane 16 places away
+// inside its group of 32 (both lanes end up with the same two values, `low` the one of the lower lane); swap_rows<32>:
+// the same between the halves of the wave.
+template <int DISTANCE>
+__device__ __forceinline__ void swap_rows(float v, float& low, float& high) {
+    const unsigned bits = __float_as_uint(v);
+    const auto swapped = DISTANCE == 16 ? __builtin_amdgcn_permlane16_swap(bits, bits, false, false)
+                                        : __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    low = __uint_as_float(static_cast<unsigned>(swapped[0]));
+    high = __uint_as_float(static_cast<unsigned>(swapped[1]));
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp32(float v) {
+    return __uint_as_float(static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(__float_as_uint(v)), CTRL, 0xF, 0xF, false)));
+}
+
+// Lane 0 of a 32-lane shuffle-down tree, offsets 16, 8, 4, 2, 1 (v[i] + v[i + offset] at every step, the order of
+// additions the reference's reduction has), in every lane of the group of 32.  Only the lanes that feed lane 0 hold
+// the tree's values on the way, which is all the result needs.
 __device__ __forceinline__ float tree32_sum(float v) {
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) v = v + __shfl_down(v, offset, 32);
-    return __shfl(v, 0, 32);
+    float low, high;
+    swap_rows<16>(v, low, high);
+    v = low + high;                  // lanes 0..15 of the group: v[i] + v[i + 16]
+    v = v + dpp32<0x108>(v);         // row_shl:8
+    v = v + dpp32<0x104>(v);         // row_shl:4
+    v = v + dpp32<0x102>(v);         // row_shl:2
+    v = v + dpp32<0x101>(v);         // row_shl:1
+    v = dpp32<0x150>(v);             // row_newbcast:0: lane 0 of each row of 16
+    swap_rows<16>(v, low, high);     // the lower row's value in both rows of the group
+    return low;
+}
+// Largest value of each group of LANES (32 or 64) lanes, in every lane of the group.
+template <int LANES>
+__device__ __forceinline__ float group_max(float v) {
+    v = fmaxf(v, dpp32<0xB1>(v));    // lane ^ 1
+    v = fmaxf(v, dpp32<0x4E>(v));    // lane ^ 2
+    v = fmaxf(v, dpp32<0x141>(v));   // mirror inside 8 lanes
+    v = fmaxf(v, dpp32<0x140>(v));   // mirror inside 16 lanes
+    float low, high;
+    swap_rows<16>(v, low, high);
+    v = fmaxf(low, high);
+    if constexpr (LANES == 64) {
+        swap_rows<32>(v, low, high);
+        v = fmaxf(low, high);
+    }
+    return v;
 }
 
 constexpr int kTopkSlots = 32;   // experts <= 32 * kTopkSlots
@@ -225,8 +266,7 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
             cached[slot] = lane + slot * LANES >= experts ? -__builtin_inff() : v != v ? -3.402823466e+38f : v;
             maximum = fmaxf(maximum, cached[slot]);
         }
-#pragma unroll
-        for (int offset = LANES / 2; offset > 0; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset, LANES));
+        maximum = group_max<LANES>(maximum);
         float sum = 0.0f;
         if constexpr (LANES == 32) {
 #pragma unroll
@@ -246,14 +286,15 @@ __device__ __forceinline__ void topk_token(const void* logits, int dtype, int to
             // (the upper lanes run the same code on values nobody reads)
 #pragma unroll
             for (int slot = 0; slot < SLOTS; ++slot) {
-                const float other = __shfl_xor(cached[slot], 32, 64);
+                float own, other;                          // of lane l < 32: its value and that of lane l + 32
+                swap_rows<32>(cached[slot], own, other);
                 const int first = (lane & 31) + slot * 64;
                 if (first < experts) sum = sum + cached[slot];
                 if (first + 32 < experts) sum = sum + other;
             }
         }
         total = tree32_sum(sum);
-        if constexpr (LANES == 64) total = __shfl(total, 0, 64);
+        if constexpr (LANES == 64) total = __uint_as_float(static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(total)), 0)));
         // The numerators order like the probabilities (division by the common total is monotone), except that
         // numerators a few units in the last place apart may give the same probability: the bound below is taken
         // on the numerators and lowered by that much, the probabilities themselves are computed for candidates only.
