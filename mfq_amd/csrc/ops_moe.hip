@@ -105,9 +105,12 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
     v = step(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, false)));
     v = step(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x141, 0xF, 0xF, false)));
     v = step(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x140, 0xF, 0xF, false)));
-    v = step(v, static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 16, kWave)));
-    v = step(v, static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 32, kWave)));
-    return v;
+    // across the rows of 16 lanes and the halves of the wave: register swaps leave the lane's value and its partner's
+    // in the two results
+    const auto rows = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    v = step(static_cast<uint32_t>(rows[0]), static_cast<uint32_t>(rows[1]));
+    const auto halves = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return step(static_cast<uint32_t>(halves[0]), static_cast<uint32_t>(halves[1]));
 }
 
 // hidden = swiglu(gate, up) of one routed pair, computed by the block that multiplies it: two columns per thread, the

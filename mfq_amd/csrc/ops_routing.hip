@@ -1139,12 +1139,20 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_pairs_kernel(PlanArgs
         const uint32_t mine = keys[s][p];
         int smaller = 0;
         const int begin = part * chunk, end = begin + chunk < P ? begin + chunk : P;
-        for (int q = begin; q < end; q += 4) {
-            const uint4 v = *reinterpret_cast<const uint4*>(&keys[s][q]);
-            smaller += (v.x < mine) + (v.y < mine) + (v.z < mine) + (v.w < mine);
+        auto below = [mine](const uint4& v) { return (v.x < mine) + (v.y < mine) + (v.z < mine) + (v.w < mine); };
+        int q = begin;
+        // sixteen keys at a time while they last, their four LDS reads requested together: one read per turn of the loop
+        // is one round trip per four keys, and a thread scans up to 128 of them
+        for (; q + 16 <= end; q += 16) {
+            const uint4* from = reinterpret_cast<const uint4*>(&keys[s][q]);
+            const uint4 v0 = from[0], v1 = from[1], v2 = from[2], v3 = from[3];
+            smaller += below(v0) + below(v1) + below(v2) + below(v3);
         }
-        // the parts of an item sit in neighbouring lanes
-        for (int step = 1; step < parts; step *= 2) smaller += __shfl_xor(smaller, step, 64);
+        for (; q < end; q += 4) smaller += below(*reinterpret_cast<const uint4*>(&keys[s][q]));
+        // the parts of an item sit in neighbouring lanes (2, 4 or 8 of them): data-parallel moves, no LDS round trip
+        if (parts > 1) smaller += __builtin_amdgcn_update_dpp(0, smaller, 0xB1, 0xF, 0xF, false);    // lane ^ 1
+        if (parts > 2) smaller += __builtin_amdgcn_update_dpp(0, smaller, 0x4E, 0xF, 0xF, false);    // lane ^ 2
+        if (parts > 4) smaller += __builtin_amdgcn_update_dpp(0, smaller, 0x141, 0xF, 0xF, false);   // the other quad of eight lanes
         if (live && part == 0) {
             const int4 record = records[s][p];
             x.pair_items[static_cast<int64_t>(s) * P + smaller] = PairItem{record.x, record.y, record.z, record.w};
