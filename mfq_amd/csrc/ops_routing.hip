@@ -553,8 +553,11 @@ __device__ __forceinline__ void wave_range(int pairs, int waves, int wave, int b
 // order, the per-pair records where asked for, and the byte and expert totals.  One block of kPlanThreads threads;
 // cnt[e], start[e] (LDS) hold the pairs of expert e and where they begin in ids_dst.  scratch [kWaves], wave_items and
 // wave_tiles [K_CLASS_COUNT][kWaves], totals [8] are LDS work arrays; lds is the base of the block's dynamic LDS.
+// The block builds the lists of slots [slot_lo, slot_hi).  `whole`: these are all the slots of the plan and the block
+// stores the totals itself; otherwise the blocks of the other slots run beside it, each adds its bytes to the total
+// (zeroed by the kernel in front) and the block of slot 0 stores the expert count.
 __device__ __forceinline__ void plan_work_lists(const PlanArgs& a, int* lds, int* cnt, int* start, int* scratch, int* wave_items,
-                                                int* wave_tiles, int* totals) {
+                                                int* wave_tiles, int* totals, int slot_lo, int slot_hi, bool whole) {
     const int E = a.experts;
     constexpr int kWaves = kPlanThreads / 64;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -570,7 +573,7 @@ __device__ __forceinline__ void plan_work_lists(const PlanArgs& a, int* lds, int
     const int my_tiles = active ? (cnt[tid] + x.prefill_tile_m - 1) / x.prefill_tile_m : 0;
     if (tid == 0) { *total_bytes = 0ull; *total_distinct = 0; }
     unsigned long long my_bytes = 0ull;
-    for (int s = 0; s < x.slots; ++s) {
+    for (int s = slot_lo; s < slot_hi; ++s) {
         lds_barrier();
         int my_pool = -1;
         ExpertInfo info{-1, 0, -1, 0, 0};
@@ -668,7 +671,15 @@ __device__ __forceinline__ void plan_work_lists(const PlanArgs& a, int* lds, int
         }
     }
     __syncthreads();
-    if (tid == 0) { *x.touched_bytes = static_cast<int64_t>(*total_bytes); *x.distinct = *total_distinct; }
+    if (tid == 0) {
+        if (whole) {
+            *x.touched_bytes = static_cast<int64_t>(*total_bytes);
+            *x.distinct = *total_distinct;
+        } else {
+            atomicAdd(reinterpret_cast<unsigned long long*>(x.touched_bytes), *total_bytes);
+            if (slot_lo == 0) *x.distinct = *total_distinct;
+        }
+    }
 }
 
 // Second kernel of a large plan: block b places the pairs of wave range b of route_plan_kernel, split
@@ -681,8 +692,9 @@ __global__ void __launch_bounds__(kPlanThreads) route_scatter_kernel(PlanArgs a)
     int* hist = lds;                    // [kWaves][E]: counts, then pairs placed so far
     int* base = hist + kWaves * E;      // [kWaves][E]: start of the run of (wave, expert)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (blockIdx.x == kWaves) {
-        // the block behind the placing ones: the work lists, from the counts and bounds route_plan_kernel left
+    if (blockIdx.x >= kWaves) {
+        // the blocks behind the placing ones: the work lists of one slot each, from the counts and bounds route_plan_kernel left
+        const int slot = blockIdx.x - kWaves;
         int* cnt = lds;
         int* start = cnt + E;
         int* scratch = start + E;
@@ -690,7 +702,13 @@ __global__ void __launch_bounds__(kPlanThreads) route_scatter_kernel(PlanArgs a)
         int* wave_tiles = wave_items + K_CLASS_COUNT * kWaves;
         int* totals = wave_tiles + K_CLASS_COUNT * kWaves;
         if (tid < E) { cnt[tid] = a.counts[tid]; start[tid] = a.expert_bounds[tid]; }
-        plan_work_lists(a, lds, cnt, start, scratch, wave_items, wave_tiles, totals);
+        if (slot >= a.lists_in_scatter) {
+            // spare blocks: the part of the activation copies that route_plan_kernel's spare blocks left
+            const int64_t item = a.tiles.first_item + static_cast<int64_t>(slot - a.lists_in_scatter) * kPlanThreads + threadIdx.x;
+            tile_pack_item(item, a.tiles.src, a.tiles.dtype, a.tiles.rows, a.tiles.width, a.tiles.layouts, a.tiles.dst, a.tiles.layout_stride);
+            return;
+        }
+        plan_work_lists(a, lds, cnt, start, scratch, wave_items, wave_tiles, totals, slot, slot + 1, a.extras.slots == 1);
         return;
     }
     int block_lo, block_hi, lo, hi;
@@ -719,7 +737,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
     extern __shared__ int lds[];
     if (blockIdx.x > 0 && a.tiles.src != nullptr) {
         // blocks behind the first copy the activations into the pair layouts of the tile kernel while the first builds the plan
-        const int64_t item = static_cast<int64_t>(blockIdx.x - 1) * kPlanThreads + threadIdx.x;
+        const int64_t item = a.tiles.first_item + static_cast<int64_t>(blockIdx.x - 1) * kPlanThreads + threadIdx.x;
         tile_pack_item(item, a.tiles.src, a.tiles.dtype, a.tiles.rows, a.tiles.width, a.tiles.layouts, a.tiles.dst, a.tiles.layout_stride);
         return;
     }
@@ -779,8 +797,12 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_kernel(PlanArgs a) {
 
     const PlanExtras& x = a.extras;
     if (x.items == nullptr) return;
-    if (a.wave_base != nullptr && a.lists_in_scatter) return;      // the block behind route_scatter_kernel's builds them meanwhile
-    plan_work_lists(a, lds, cnt, start, scratch, wave_items, wave_tiles, totals);
+    if (a.wave_base != nullptr && a.lists_in_scatter) {
+        // the blocks behind route_scatter_kernel's build them meanwhile, one per slot, and add up the byte total
+        if (tid == 0 && x.slots > 1) *x.touched_bytes = 0;
+        return;
+    }
+    plan_work_lists(a, lds, cnt, start, scratch, wave_items, wave_tiles, totals, 0, x.slots, true);
 }
 
 // The same plan for at most kPlanThreads pairs (decode): one thread per pair and per expert, no
@@ -1282,24 +1304,30 @@ void launch_route_plan(const PlanArgs& args, hipStream_t stream) {
     MFQ_REQUIRE(args.route.logits == nullptr, "fused routing needs a decode-sized plan");
     MFQ_REQUIRE(args.wave_base == nullptr || args.extras.pair_items == nullptr, "per-pair records need the one-kernel plan");
     int spare_blocks = pack_rows;
+    int later_blocks = 0;      // of the activation copies, left to the spare blocks of the scatter launch
     if (args.tiles.src != nullptr) {
         MFQ_REQUIRE(pack_rows == 0 && args.tiles.dst != nullptr && args.tiles.width % dev::kLaneColumns == 0 && args.tiles.dtype != MFQ_AMD_F32 &&
                         reinterpret_cast<uintptr_t>(args.tiles.src) % 16 == 0,
                     "activations cannot be copied into the tile layouts by the plan kernel");
         const int64_t items = static_cast<int64_t>(args.tiles.rows) * (args.tiles.width / dev::kLaneColumns);
         spare_blocks = static_cast<int>((items + kPlanThreads - 1) / kPlanThreads);
+        // The copies move more bytes than the plan block takes time for (four layouts of 4096 x 2048: 80 MB, 34 us
+        // against 21), and the scatter launch leaves most of the chip idle too: it takes half of them.
+        if (args.wave_base != nullptr && args.extras.items != nullptr) { later_blocks = spare_blocks / 2; spare_blocks -= later_blocks; }
     }
-    // with a scatter launch behind it, the plan kernel stops after the bounds; the work lists are built by one more
-    // block of the scatter launch, beside the blocks that place the pairs
+    // with a scatter launch behind it, the plan kernel stops after the bounds; the work lists are built by more blocks
+    // of the scatter launch, one per slot, beside the blocks that place the pairs
     PlanArgs large_args = args;
-    large_args.lists_in_scatter = args.wave_base != nullptr && args.extras.items != nullptr ? 1 : 0;
+    large_args.lists_in_scatter = args.wave_base != nullptr && args.extras.items != nullptr ? args.extras.slots : 0;
+    large_args.tiles.first_item = 0;
     hipLaunchKernelGGL(dev::route_plan_kernel, dim3(1 + spare_blocks), dim3(kPlanThreads), lds, stream, large_args);
     check_launch("route_plan_kernel");
     if (args.wave_base != nullptr) {
         const size_t place_lds = sizeof(int) * 2 * (kPlanThreads / 64) * args.experts;
         const size_t scatter_lds = place_lds > lds ? place_lds : lds;       // the lists block lays its LDS out as the plan kernel does
         if (scatter_lds > 64 * 1024) (void)device_state();
-        hipLaunchKernelGGL(dev::route_scatter_kernel, dim3(kPlanThreads / 64 + large_args.lists_in_scatter), dim3(kPlanThreads), scatter_lds,
+        large_args.tiles.first_item = static_cast<int64_t>(spare_blocks) * kPlanThreads;
+        hipLaunchKernelGGL(dev::route_scatter_kernel, dim3(kPlanThreads / 64 + large_args.lists_in_scatter + later_blocks), dim3(kPlanThreads), scatter_lds,
                            stream, large_args);
         check_launch("route_scatter_kernel");
     }

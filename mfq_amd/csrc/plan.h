@@ -105,6 +105,7 @@ struct PlanTilePack {
     int64_t layout_stride;
     int32_t rows, width, dtype;
     uint32_t layouts;       // bit l: layout l is wanted
+    int64_t first_item;     // set by the launcher: the lane block (row * width / 32 + block) the launch's spare blocks start at
 };
 
 // Router logits to select the routes from inside the plan kernel (decode only), or logits == null.
@@ -130,7 +131,7 @@ struct PlanArgs {
     PlanExtras extras;        // extras.items == nullptr: plain route plan
     PlanPack pack;
     PlanTilePack tiles;
-    int32_t lists_in_scatter;   // large plans (set by the launcher): the work lists are built by a block of the scatter launch
+    int32_t lists_in_scatter;   // large plans (set by the launcher): the work lists are built by blocks of the scatter launch, one per slot
     PlanRoute route;
 };
 
