@@ -469,6 +469,7 @@ void launch_rows_fast(const RowsArgs& args, int slots, bool nvq, hipStream_t str
         if (narrow) {
             if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 4>);
             else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 8>);
+            else if (wave_slots == 16) launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 16>);
             else launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 0>);
         } else {
             if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<64, dev::kXPacked, 4>);
@@ -922,15 +923,17 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         const int active_bound = pairs < E ? pairs : E;
         int rows_in_width = 0;
         // Enough blocks to fill the chip at small batches, long row runs per wave at large ones: the tallest block with
-        // straight-line code (16 row slots per wave for wide rows, 8 for rows of at most 512 columns), halved while the
+        // straight-line code (16 row slots per wave: 64 rows of more than 512 columns, 256 rows of at most 512, about
+        // 64 KB of packed rows either way; the down blocks that compute their own hidden row have 8), halved while the
         // launch has fewer blocks than the chip holds at once (measured at 512 experts x (2048 <-> 512), top-10: a floor
         // of 1024 blocks against 2048 gives 41.9 vs 43.1 us per step at batch 4 and 57.2 vs 60.1 us at batch 8, and
-        // leaves batches 1, 2 and 16 where they were; 512 is slower everywhere)
+        // leaves batches 1, 2 and 16 where they were; 512 is slower everywhere.  At batch 16 the down launch takes
+        // 22.7 us with 256 rows per block against 23.7 with 128; gate+up with 128 rows per block 39.8 against 38.7)
         auto rows_per_block = [&](int out_rows, int slots) {
             const int least = rows_fast_min_block(rows_in_width);
-            int rows = rows_in_width <= 16 * dev::kLaneColumns ? 128 : 64;
-            while (rows > least && static_cast<int64_t>(pairs) * slots * ((out_rows + rows - 1) / rows) < 1024) rows /= 2;
-            return rows;
+            int height = rows_in_width > 16 * dev::kLaneColumns ? 64 : rows.gu != nullptr ? 128 : 256;
+            while (height > least && static_cast<int64_t>(pairs) * slots * ((out_rows + height - 1) / height) < 1024) height /= 2;
+            return height;
         };
         auto run_rows = [&](int slot_lo, int slot_hi) {
             const int slots = slot_hi - slot_lo;
