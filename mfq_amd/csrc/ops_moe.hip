@@ -401,7 +401,9 @@ __global__ void shared_expert_reduce_kernel(const uint16_t* pairs, const float* 
 }  // namespace dev
 
 namespace {
-constexpr int kFusedSwigluPairs = 100;   // up to this many routed pairs the down blocks compute their hidden rows themselves
+// The down blocks compute the hidden row of their pair themselves up to this many routed pairs, or, beyond that, up to
+// this many down blocks per pair (every block of a pair repeats the SwiGLU of its row).
+constexpr int kFusedSwigluPairs = 100, kFusedSwigluBlocks = 8;
 
 void launch_weighted_reduce(const uint16_t* pairs, const float* weights, const int32_t* ids, int experts, int tokens, int top_k,
                             int width, void* out, int out_dtype, hipStream_t stream) {
@@ -463,6 +465,7 @@ void launch_rows_fast(const RowsArgs& args, int slots, bool nvq, hipStream_t str
         MFQ_REQUIRE(narrow && args.in_per_pair && args.sigmoid != nullptr, "the fused SwiGLU serves rows of at most 512 columns");
         if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 4>);
         else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 8>);
+        else if (wave_slots == 16) launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 16>);
         else launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 0>);
     } else if (args.in_packed != nullptr) {
         // straight-line variants for the block heights the FFN uses, the looped kernel for the rest
@@ -869,10 +872,13 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         const bool fast_mode = decode && f->config.launch_mode == 0;
         const bool pack_x = fast_mode && f->d_x_packed != nullptr;
         // the down blocks compute the hidden row of their pair themselves when nothing else reads it
-        // (every block of a pair repeats the SwiGLU and the packing of its row: worth a kernel less up to about a hundred
-        // pairs; measured at 512 experts x (2048 <-> 512), top-10: batch 1 -4 us, batch 4 -5 us per step, batch 16 +0.5 us)
+        // (every block of a pair repeats the SwiGLU and the packing of its row: a kernel less against that.  Measured at
+        // 512 experts x (2048 <-> 512), top-10, per step: batch 1 -4 us, batch 4 -5 us; batch 16 +0.5 us with sixteen
+        // down blocks per pair and -2.7 us with eight, batch 32 -3.1 us with eight)
+        int down_height = 256;     // as rows_per_block() below will choose it for the down launch
+        while (down_height > 64 && static_cast<int64_t>(pairs) * ((H + down_height - 1) / down_height) < 1024) down_height /= 2;
         const bool fuse_swiglu = fast_mode && !f->decode_needs_items && I <= 16 * dev::kLaneColumns && rows_fast_geometry(I, MFQ_AMD_F16) &&
-                                 pairs <= kFusedSwigluPairs;
+                                 (pairs <= kFusedSwigluPairs || (H + down_height - 1) / down_height <= kFusedSwigluBlocks);
         const bool pack_hidden = fast_mode && !fuse_swiglu && f->d_hidden_packed != nullptr;
         if (pack_x) {
             plan.pack.src = x_dev; plan.pack.dst = f->d_x_packed; plan.pack.stride = dev::xpack_row_dwords(H);
@@ -924,14 +930,14 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         int rows_in_width = 0;
         // Enough blocks to fill the chip at small batches, long row runs per wave at large ones: the tallest block with
         // straight-line code (16 row slots per wave: 64 rows of more than 512 columns, 256 rows of at most 512, about
-        // 64 KB of packed rows either way; the down blocks that compute their own hidden row have 8), halved while the
+        // 64 KB of packed rows either way), halved while the
         // launch has fewer blocks than the chip holds at once (measured at 512 experts x (2048 <-> 512), top-10: a floor
         // of 1024 blocks against 2048 gives 41.9 vs 43.1 us per step at batch 4 and 57.2 vs 60.1 us at batch 8, and
         // leaves batches 1, 2 and 16 where they were; 512 is slower everywhere.  At batch 16 the down launch takes
         // 22.7 us with 256 rows per block against 23.7 with 128; gate+up with 128 rows per block 39.8 against 38.7)
         auto rows_per_block = [&](int out_rows, int slots) {
             const int least = rows_fast_min_block(rows_in_width);
-            int height = rows_in_width > 16 * dev::kLaneColumns ? 64 : rows.gu != nullptr ? 128 : 256;
+            int height = rows_in_width > 16 * dev::kLaneColumns ? 64 : 256;
             while (height > least && static_cast<int64_t>(pairs) * slots * ((out_rows + height - 1) / height) < 1024) height /= 2;
             return height;
         };
