@@ -178,7 +178,8 @@ def test_many_pairs_per_expert_and_large_activations():
         assert np.isfinite(expect[t]).all() and rel_l2(out[t], expect[t]) <= FFN_TOL, t
 
 
-@pytest.mark.parametrize("tokens,experts,k", [(1, 24, 6), (16, 24, 6), (32, 128, 8), (5, 256, 8), (3, 8, 2), (40, 24, 6)])
+@pytest.mark.parametrize("tokens,experts,k", [(1, 24, 6), (16, 24, 6), (32, 128, 8), (5, 256, 8), (3, 8, 2), (40, 24, 6),
+                                                (13, 40, 4), (9, 512, 10)])
 def test_layer_with_fused_routing_equals_topk_then_layer(tokens, experts, k):
     """run_logits selects the routes inside the plan kernel (up to 32 tokens; 40 takes the top-k kernel):
     ids bit-equal to the stand-alone top-k, weights and output equal to the two-call sequence."""
