@@ -158,6 +158,23 @@ def test_layer_with_the_4096_entry_e8_profile(tokens):
     assert rel_l2(out, oracle_layer(x, ids, weights, tensors)) <= FFN_TOL
 
 
+def test_tall_down_blocks_beside_pools_of_the_exact_kernels():
+    """32 tokens x top-4 over 2048 outputs: 128 pairs x 8 down blocks of 256 rows reach the floor of the launch, and
+    a pool that only the exact kernels serve keeps the SwiGLU in a kernel of its own, so the streaming pools run
+    the sixteen-slot rows kernel on packed hidden rows."""
+    import torch
+    from mfq_amd import runtime as R
+    experts, hidden, inter, k, tokens = 12, 2048, 96, 4, 32
+    mix = (("NVQ2J-XL", 0.3), ("NINT4", 0.25), ("NVQ3J-L", 0.2), ("NINT3", 0.15), ("MXFP4", 0.1))
+    tensors, runtimes, formats = _layer("test/moe/tall-down", experts, hidden, inter, "random", mix=mix)
+    assert any("NVQ2J-XL" in f for f in formats) and len(set(sum(formats, []))) >= 3
+    x, ids, weights = _inputs("test/moe/tall-down/in", tokens, experts, hidden, k)
+    ffn = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens)
+    out = ffn.run(torch.from_numpy(x).to(torch.bfloat16).cuda(), torch.from_numpy(ids).cuda(),
+                  torch.from_numpy(weights).cuda()).cpu().numpy()
+    assert rel_l2(out, oracle_layer(x, ids, weights, tensors)) <= FFN_TOL
+
+
 def test_many_pairs_per_expert_and_large_activations():
     """32 tokens over 6 experts: every expert serves many pairs; per-token activation scales from
     2^-3 to 2^5 exercise the per-token normalisation of the streaming kernels (larger inputs overflow
