@@ -464,6 +464,91 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         }
         __syncthreads();
     };
+    // The same step as a software pipeline (packed activations): while the MFMAs of chunk j run, the weights of
+    // chunk j + 1 are decoded and its activation operands read from LDS, so that the matrix pipe, the vector pipe
+    // and the LDS work at the same time inside one wave.  The first chunk of a step is decoded during the last
+    // chunk of the step before it (`block`, `wq` carry it across the barrier).  The order of the instructions of a
+    // chunk is prescribed to the scheduler: one MFMA, an LDS read, a share of the vector instructions.
+    WeightBlock<CLS> block[2];
+    uint32_t wq[2][4];
+    auto a_read = [&](int step, int j, half8_t (&av)[MT]) {
+        const unsigned char* x_tile = x_lds + (step & 1) * kFastXBytes;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) av[mt] = *reinterpret_cast<const half8_t*>(x_tile + mt * 32 * 128 + a_piece[mt & 1][j]);
+    };
+    auto decode_first = [&](int step, const FastRaw<CLS> (&raw)[2]) {
+        const int last = steps - 1;
+        const LaneBlock b = lane_block<C::kGs>(2 * (step < last ? step : last) + h, width, ctx.groups);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            uint32_t scales = 0, minima = 0;
+            if constexpr (C::kNint) { scales = level_pair(0, t, b); minima = level_pair(1, t, b); }
+            if constexpr (C::kNvq) side_pair(t, b, scales, minima);
+            block[t] = weight_block<CLS>(ctx, b, raw[t], scale[t], scales, minima);
+            chunk_weights<CLS, IB>(block[t], raw[t], 0, wq[t]);
+        }
+    };
+    // vector instructions of one chunk of two rows, roughly: what the scheduler spreads between the MFMAs
+    constexpr int kChunkValu = C::kNvq ? 72 : C::kMx ? 12 : C::kBits == 3 ? 40 : 32;
+    // ... and of the last chunk of a step, which also sets up the next step's lane blocks and requests packed rows
+    constexpr int kLastValu = kChunkValu + (C::kNint ? 72 : C::kNvq ? 56 : 20);
+    auto step_piped = [&](int step, FastRaw<CLS> (&raw)[2], const FastRaw<CLS> (&raw_next)[2]) {
+        half8_t aq[MT];
+        a_read(step, 0, aq);
+        x_direct(step + 1 < steps ? step + 1 : steps - 1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            __builtin_amdgcn_sched_barrier(0);
+            uint32_t wn[2][4];
+            half8_t an[MT];
+            const half8_t b0 = as_half8(wq[0][0], wq[0][1], wq[0][2], wq[0][3]);
+            const half8_t b1 = as_half8(wq[1][0], wq[1][1], wq[1][2], wq[1][3]);
+            if (j < 3) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) chunk_weights<CLS, IB>(block[t], raw[t], j + 1, wn[t]);
+                a_read(step, j + 1, an);
+            } else {
+                // every chunk of this step is decoded: the packed registers take the step after next, and the
+                // first chunk of the next step is decoded from the other ring slot (into wq: b0 and b1 hold this chunk)
+                fetch(step + 2, raw);
+                decode_first(step + 1, raw_next);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                acc[0][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq[mt], b0, acc[0][mt], 0, 0, 0);
+                acc[1][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aq[mt], b1, acc[1][mt], 0, 0, 0);
+            }
+            constexpr int kShare = (kChunkValu + 2 * MT - 1) / (2 * MT), kLastShare = (kLastValu + 2 * MT - 1) / (2 * MT);
+            if (j < 3) {
+#pragma unroll
+                for (int i = 0; i < 2 * MT; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        // an LDS read
+                    __builtin_amdgcn_sched_group_barrier(0x002, kShare, 0);   // vector instructions
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 2 * MT; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);        // a request for packed rows
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, kLastShare, 0);
+                }
+            }
+            if (j < 3) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) wq[t][m] = wn[t][m];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) aq[mt] = an[mt];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // this wave's direct loads have landed; only the weight loads issued after them may be pending
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * fetch_loads<CLS>()) : "memory");
+        __syncthreads();
+    };
     const int run = C::kNvq ? side_run : level_run;
     for (int from = 0; from < steps; from += run) {
         // every wave is past the last step of the previous run (its closing barrier) when the window moves
@@ -471,9 +556,17 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         if constexpr (C::kNvq) stage_side(from);
         __syncthreads();
         const int to = from + run < steps ? from + run : steps;
-        for (int step = from; step < to; step += 2) {
-            step_body(step, ring[0]);
-            step_body(step + 1, ring[1]);
+        if constexpr (PACKED) {
+            decode_first(from, ring[0]);     // `from` is even: the run's first step reads ring slot 0
+            for (int step = from; step < to; step += 2) {
+                step_piped(step, ring[0], ring[1]);
+                step_piped(step + 1, ring[1], ring[0]);
+            }
+        } else {
+            for (int step = from; step < to; step += 2) {
+                step_body(step, ring[0]);
+                step_body(step + 1, ring[1]);
+            }
         }
     }
 
