@@ -244,6 +244,10 @@ int mfq_amd_moe_ffn_run_router(mfq_amd_moe_ffn* ffn, const void* x_dev, const vo
                                int32_t normalize, float norm_floor, float scale, int32_t tokens, void* out_dev, void* stream);
 /* Routes of the last mfq_amd_moe_ffn_run_logits: ids i32 [tokens, k], weights f32 [tokens, k]. */
 int mfq_amd_moe_ffn_routes(mfq_amd_moe_ffn* ffn, const int32_t** ids_dev, const float** weights_dev);
+/* Which projections (bit 0 gate, bit 1 up, bit 2 down) have their MXFP4 prefill tiles on the block-scaled MFMA.  create
+ * honours mx_scaled_mfma = 1 only for 16-bit activations, launch_mode 0, max_tokens above the decode limit and widths the
+ * streaming tile kernel serves; this says what it decided.  No counterpart in the reference. */
+int mfq_amd_moe_ffn_mx_scaled_slots(mfq_amd_moe_ffn* ffn, int32_t* mask);
 /* Stage buffers of the last run (device pointers, valid until destroy): gate_up f16 [tokens, k, 2, I]
  * (gate then up), pairs f16 [tokens, k, H]. */
 int mfq_amd_moe_ffn_buffers(mfq_amd_moe_ffn* ffn, const void** gate_up_f16, const void** pairs_f16);

@@ -86,6 +86,7 @@ EXPORTS = {
     "mfq_amd_moe_ffn_run_shared": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                             C.c_void_p, C.c_void_p]),
     "mfq_amd_moe_ffn_routes": (C.c_int, [C.c_void_p, c_void_pp, c_void_pp]),
+    "mfq_amd_moe_ffn_mx_scaled_slots": (C.c_int, [C.c_void_p, C.POINTER(C.c_int32)]),
     "mfq_amd_moe_ffn_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p,
                                       C.c_void_p]),
     "mfq_amd_moe_ffn_buffers": (C.c_int, [C.c_void_p, c_void_pp, c_void_pp]),

@@ -65,6 +65,14 @@ __device__ __forceinline__ uint16_t float_to_half_bits(float v) {
     return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));   // round to nearest even
 }
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return bits_to_float(static_cast<uint32_t>(b) << 16); }
+// half(a * b) with the product rounded to fp32 first, as the reference's __float2half(a * b).  float_to_half_bits(a * b)
+// is not that for every input: the compiler fuses the multiply into the conversion as v_fma_mixlo_f16 a, b, +0, and the
+// +0 addend turns a product of -0 (a gate of -0.0) into +0.  The empty statement keeps the two apart.
+__device__ __forceinline__ uint16_t product_to_half_bits(float a, float b) {
+    float product = a * b;
+    asm("" : "+v"(product));
+    return float_to_half_bits(product);
+}
 
 // exp() of the routing softmax and of the shared-expert gate, defined operation by operation so that any IEEE machine
 // produces the same bits: n = rint(x*log2e); r = x - n*ln2 in two fma steps; degree-5 Horner
@@ -110,11 +118,11 @@ __device__ __forceinline__ uint16_t swiglu_bits(uint16_t gb, uint16_t ub, float 
     if (limit > 0.0f) {
         const float clipped = fminf(g, limit);
         const float value = fminf(fmaxf(u, -limit), limit);
-        return float_to_half_bits((clipped / (1.0f + expf(-clipped))) * value);
+        return product_to_half_bits(clipped / (1.0f + expf(-clipped)), value);
     }
     const float sigmoid = half_bits_to_float(table[gb]);
-    const float first = half_bits_to_float(float_to_half_bits(g * sigmoid));
-    return float_to_half_bits(first * u);
+    const float first = half_bits_to_float(product_to_half_bits(g, sigmoid));
+    return product_to_half_bits(first, u);
 }
 
 // ---------------------------------------------------------------- NINT ----

@@ -865,10 +865,8 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         x.touched_bytes = f->d_touched; x.distinct = f->d_distinct;
         x.tile_capacity = f->tile_capacity; x.prefill_tile_m = kPrefillTileM; x.want_tiles = decode ? 0 : 1;
         x.want_items = !decode || f->decode_needs_items;
-        // up to four tokens: experts rarely repeat, so nothing is gained by sorting the pairs by expert
         // a streaming decode step needs nothing but the pair lists
         x.pairs_only = decode && !x.want_items && f->config.launch_mode == 0 && pairs <= kPlanSortPairs;
-        x.direct_pairs = !x.pairs_only && decode && tokens <= 4 && !x.want_items && f->d_expert_info != nullptr && f->config.launch_mode == 0;
         const bool fast_mode = decode && f->config.launch_mode == 0;
         const bool pack_x = fast_mode && f->d_x_packed != nullptr;
         // the down blocks compute the hidden row of their pair themselves when nothing else reads it
@@ -951,7 +949,10 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
                     for (int s = slot_lo; s < slot_hi; ++s) { nvq = nvq || f->tables.fast_nvq[s]; mx = mx || f->mx_scaled[s]; }
                     mx = mx && f->d_fp8 != nullptr;
                     if (mx) {
-                        // MXFP4 tiles on the block-scaled MFMA: the activations of the stage as E4M3 terms first
+                        // MXFP4 tiles on the block-scaled MFMA: the activations of the stage as E4M3 terms first.  The
+                        // split reads its rows in plain column order; hidden rows written for the tile kernel are in the
+                        // layout of their down pool's class, which for MXFP4 must therefore be the plain one.
+                        MFQ_REQUIRE(tile_layout_of_class(dev::K_MXFP4) == 2, "the E4M3 split reads MXFP4 rows in column order");
                         const int terms = rows.in_dtype == MFQ_AMD_BF16 ? 2 : 3;
                         launch_fp8_split(rows.in, rows.in_dtype, rows.in_per_pair ? pairs : tokens, rows.in_width, terms, f->d_fp8,
                                          f->d_fp8_scales, stream);
@@ -1141,6 +1142,15 @@ extern "C" int mfq_amd_moe_ffn_routes(mfq_amd_moe_ffn* f, const int32_t** ids_de
         MFQ_REQUIRE(f, "null argument");
         if (ids_dev) *ids_dev = f->d_route_ids;
         if (weights_dev) *weights_dev = f->d_route_weights;
+    });
+}
+
+extern "C" int mfq_amd_moe_ffn_mx_scaled_slots(mfq_amd_moe_ffn* f, int32_t* mask) {
+    return guarded([&] {
+        MFQ_REQUIRE(f && mask, "null argument");
+        *mask = 0;
+        for (int s = 0; s < kSlots; ++s)
+            if (f->mx_scaled[s] && f->d_fp8) *mask |= 1 << s;
     });
 }
 
@@ -1351,6 +1361,8 @@ extern "C" int mfq_amd_grouped_matmul_static(const mfq_amd_moe_tensor* tensor, c
     return guarded([&] {
         MFQ_REQUIRE(tensor, "null argument");
         MFQ_REQUIRE(tokens >= 0 && top_k >= 1 && tensor->experts > 0, "invalid route geometry");
+        MFQ_REQUIRE(tensor && tokens >= 0 && top_k >= 1 && tensor->experts > 0 && tensor->experts <= kPlanMaxExperts,
+                    "invalid route geometry");
         const int64_t needed = mfq_amd_grouped_matmul_workspace(tokens, top_k, tensor->experts);
         if (needed > kStaticScratchBytes)
             fail_invalid("route plan of " + std::to_string(needed) + " bytes exceeds the static scratch of " +

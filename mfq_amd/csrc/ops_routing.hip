@@ -840,12 +840,11 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_small_kernel(PlanArgs
     constexpr int kWaves = kPlanThreads / 64;
     const PlanExtras& x = a.extras;
 
-    const bool direct = x.items != nullptr && x.direct_pairs != 0;
     // issued first, consumed last: the per-expert records of every slot
     ExpertInfo info[kSlots];
 #pragma unroll
     for (int s = 0; s < kSlots; ++s)
-        info[s] = !direct && x.items != nullptr && x.expert_info != nullptr && s < x.slots && tid < E ? x.expert_info[s * E + tid]
+        info[s] = x.items != nullptr && x.expert_info != nullptr && s < x.slots && tid < E ? x.expert_info[s * E + tid]
                                                                                                        : ExpertInfo{-1, 0, -1, 0, 0};
     int expert = -1;
     if (TOPK_SLOTS > 0) {
@@ -868,36 +867,6 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_small_kernel(PlanArgs
     } else {
         if (tid < P) { expert = a.ids[tid]; if (static_cast<unsigned>(expert) >= static_cast<unsigned>(E)) expert = -1; }
         expert_of[tid] = expert;
-    }
-    if (direct) {
-        // A handful of pairs: every pair looks up its expert's records itself and the list stays in pair order.
-        // cnt doubles as the set of experts seen so far (one bit each) for the byte and expert counts.
-        if (tid < (E + 31) / 32) cnt[tid] = 0;
-        if (tid == 0) { total_bytes = 0ull; total_distinct = 0; }
-        __syncthreads();
-        if (tid < P) {
-            bool first = false;
-            if (expert >= 0) {
-                const unsigned bit = 1u << (expert & 31);
-                first = (static_cast<unsigned>(atomicOr(&cnt[expert >> 5], static_cast<int>(bit))) & bit) == 0u;
-            }
-            unsigned long long bytes = 0ull;
-            for (int s = 0; s < x.slots; ++s) {
-                PairItem item{-1, 0, 0, -1};
-                if (expert >= 0) {
-                    const ExpertInfo record = x.expert_info[s * E + expert];
-                    if (record.pool >= 0) {
-                        item = PairItem{tid, record.pool, record.local, record.cls};
-                        bytes += static_cast<unsigned long long>(record.bytes);
-                    }
-                }
-                x.pair_items[static_cast<int64_t>(s) * P + tid] = item;
-            }
-            if (first) { atomicAdd(&total_bytes, bytes); atomicAdd(&total_distinct, 1); }
-        }
-        __syncthreads();
-        if (tid == 0) { *x.touched_bytes = static_cast<int64_t>(total_bytes); *x.distinct = total_distinct; }
-        return;
     }
     if (tid < E) { cnt[tid] = 0; token_mask[tid] = 0ull; }
     if (tid == 0) { total_bytes = 0ull; total_distinct = 0; repeated = 0; }
@@ -1258,10 +1227,6 @@ void launch_route_plan(const PlanArgs& args, hipStream_t stream) {
     MFQ_REQUIRE(pack_rows == 0 || (args.pack.width % dev::kLaneColumns == 0 && args.pack.width <= dev::kLaneColumns * kPlanThreads),
                 "activation width cannot be packed");
     // decode-sized plans that need no prefill tiles take the one-thread-per-pair kernel
-    MFQ_REQUIRE(!args.extras.direct_pairs ||
-                    (args.pairs <= kPlanThreads && args.extras.items != nullptr && args.extras.expert_info != nullptr &&
-                     args.extras.pair_items != nullptr && !args.extras.want_tiles && !args.extras.want_items),
-                "pair records in pair order need a decode-sized plan with resolved expert records and no other lists");
     const bool large = !args.extras.pairs_only && !(args.pairs <= kPlanThreads && (args.extras.items == nullptr || !args.extras.want_tiles));
     MFQ_REQUIRE(args.tiles.src == nullptr || large, "only the large plan kernel copies activations into the tile layouts");
     if (args.extras.pairs_only) {

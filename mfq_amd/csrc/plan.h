@@ -80,9 +80,6 @@ struct PlanExtras {
     int32_t prefill_tile_m;
     int32_t want_tiles;                // 0: tile_items / tile_offsets are not needed (decode)
     int32_t want_items;                // 0: items / item_info / class_offsets are not needed (no exact-kernel work)
-    int32_t direct_pairs;              // 1 (decode-sized plans with expert_info and without want_items / want_tiles only):
-                                       // pair_items in pair order, nothing sorted, and none of counts, expert_bounds,
-                                       // ids_dst, items written; for batches so small that experts rarely repeat
     int32_t pairs_only;                // 1 (at most kPlanSortPairs pairs, expert_info given, no want_items / want_tiles):
                                        // only pair_items is produced, by the kernel that ranks the pairs directly;
                                        // none of counts, expert_bounds, ids_dst, items, touched_bytes, distinct written

@@ -305,6 +305,12 @@ class MfeFfnRuntime:
                                                    shared_gate.data_ptr(), _dtype_code(shared_gate), tokens, out.data_ptr(), _stream()))
         return out
 
+    def mx_scaled_slots(self) -> int:
+        """Bit s set: the MXFP4 prefill tiles of projection s (gate, up, down) run on the block-scaled MFMA."""
+        mask = C.c_int32(0)
+        L.check(L.lib().mfq_amd_moe_ffn_mx_scaled_slots(self._handle, C.byref(mask)))
+        return int(mask.value)
+
     def routes(self, tokens: int) -> tuple[torch.Tensor, torch.Tensor]:
         """Copies of the ids and weights the last run_logits selected."""
         ids, weights = C.c_void_p(), C.c_void_p()

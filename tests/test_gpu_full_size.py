@@ -52,10 +52,10 @@ def _decode_inputs(tokens):
     return x, router, xd, logits
 
 
-def test_decode_batch16_vs_oracle():
+@pytest.mark.parametrize("tokens", [1, 4, 16])      # one wave per token in the plan's top-k up to 8 tokens, half a wave above
+def test_decode_batch_vs_oracle(tokens):
     from mfq_amd import runtime as R
     layer = _layer()
-    tokens = 16
     x, router, xd, logits = _decode_inputs(tokens)
     ffn = R.MfeFfnRuntime(*layer, top_k=TOP_K, max_tokens=tokens)
     out = ffn.run_logits(xd, logits).cpu().numpy()

@@ -401,6 +401,9 @@ def test_swiglu_and_reduce_ops():
     rng = np.random.default_rng(9)
     g = rng.normal(0, 2, 4096).astype(np.float16)
     u = rng.normal(0, 2, 4096).astype(np.float16)
+    # zeros of both signs and products that underflow to a zero: the sign of the zero is part of the bits
+    g[:8] = [0.0, -0.0, -6e-8, 6e-8, -1e-7, 3.0, -3.0, -0.0]
+    u[:8] = [3.0, 3.0, 2.0, -2.0, 1e-4, -0.0, 0.0, -0.0]
     got = R.swiglu(torch.from_numpy(g).cuda(), torch.from_numpy(u).cuda()).cpu().numpy()
     expect = np.array([O.lib().orc_swiglu_f16(int(a), int(b), 0.0) for a, b in zip(g.view(np.uint16), u.view(np.uint16))],
                       dtype=np.uint16)

@@ -24,6 +24,7 @@ TOL = 1e-3
     ("NINT4-32", 4096, 4096, 8), ("MXFP4", 4096, 4096, 8), ("NINT3", 4096, 2560, 9),    # two slabs, one token per block
     ("NINT4", 2048, 2048, 16), ("NVQ3J-L", 2048, 2048, 8), ("MXFP4", 2048, 1024, 16), ("NINT8", 2100, 1536, 16),
     ("NINT2", 2048, 512, 16), ("NINT4", 2050, 512, 16), ("NVQ3J-L", 2048, 512, 8), ("MXFP4", 4096, 256, 8),
+    ("NINT4-32", 4096, 4096, 1), ("NVQ3", 4096, 4096, 1),        # the two dense benchmark matrices at batch 1 (not tall)
 ])
 def test_tall_gemv_instantiations_vs_oracle(fmt, rows, width, batch):
     import torch
@@ -35,7 +36,7 @@ def test_tall_gemv_instantiations_vs_oracle(fmt, rows, width, batch):
     view = tensor.pools[0].view
     threshold = 16384 if fmt.startswith("NVQ") else 32768
     group = 2 if fmt.startswith("NVQ") and width > 2048 else 1
-    assert rows * ((batch + group - 1) // group) >= threshold, "the case must reach the tall instantiation"
+    assert batch == 1 or rows * ((batch + group - 1) // group) >= threshold, "the case must reach the tall instantiation"
     x = synth.to_bf16(synth.normal(f"test/tall/x/{width}/{batch}", (batch, width)))
     xd = torch.from_numpy(x).to(torch.bfloat16).cuda()
     y = torch.full((batch, rows), float("nan"), dtype=torch.float32, device="cuda")
@@ -64,18 +65,21 @@ def test_clamped_swiglu_operator_vs_oracle():
     for limit in (7.0, 1.5, 30.0):
         got = R.swiglu(torch.from_numpy(g).cuda(), torch.from_numpy(u).cuda(), limit).cpu().numpy()
         expect = O.swiglu_array(g, u, limit)
-        # fp16 bits on one ordered scale (the two zeros coincide)
+        # fp16 bits on one ordered scale; zeros are compared by their bits, sign included (a gate of -0.0 gives -0.0 * up)
         ordered = lambda h: np.where(h.view(np.uint16) & 0x8000, -(h.view(np.uint16) & 0x7FFF).astype(np.int32),
                                      h.view(np.uint16).astype(np.int32))
         a, b = ordered(got), ordered(expect)
         assert np.all(np.abs(a - b) <= 1), (limit, np.abs(a - b).max())
-        assert np.mean(a == b) > 0.98
+        assert np.mean(got.view(np.uint16) == expect.view(np.uint16)) > 0.98
+        zero = (expect.view(np.uint16) & 0x7FFF) == 0
+        assert zero.sum() >= 2 and np.array_equal(got.view(np.uint16)[zero], expect.view(np.uint16)[zero])
+        assert np.array_equal(got.view(np.uint16)[:6], expect.view(np.uint16)[:6])     # the six special inputs, bit for bit
         # the gate is clipped from above only, the other operand on both sides
         big = np.abs(got.astype(np.float32)).max()
         assert big <= limit * limit * 1.001
 
 
-@pytest.mark.parametrize("tokens", [3, 16, 48])     # decode kernels (direct and sorted plans) and the tile kernels
+@pytest.mark.parametrize("tokens", [3, 16, 48])     # decode kernels (one wave and half a wave per token in the plan) and the tile kernels
 def test_layer_with_clamped_swiglu_vs_oracle(tokens):
     import torch
     from mfq_amd import runtime as R
@@ -346,7 +350,7 @@ def test_prefill_mxfp4_on_the_block_scaled_mfma(case):
     elif case == "f16":
         uniform, dtype = "MXFP4", torch.float16
     else:
-        uniform, hidden, inter, tokens = "MXFP4", 96, 32, 70          # three and one lane blocks per row
+        uniform, hidden, inter, tokens = "MXFP4", 96, 160, 70         # three and five lane blocks per row: odd counts
     tensors, runtimes, formats = _layer(f"test/mxscaled/{case}", experts, hidden, inter, "random", mix=mix, uniform=uniform)
     assert any("MXFP4" in f for f in formats)
     x = synth.normal(f"test/mxscaled/x/{case}", (tokens, hidden))
@@ -355,8 +359,12 @@ def test_prefill_mxfp4_on_the_block_scaled_mfma(case):
     weights = np.full((tokens, k), 1.0 / k, dtype=np.float32)
     args = (torch.from_numpy(x).to(dtype).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(weights).cuda())
     expect = oracle_layer(x, ids, weights, tensors)
-    scaled = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens, x_dtype=dtype, mx_scaled_mfma=True).run(*args).cpu().numpy()
-    plain = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens, x_dtype=dtype).run(*args).cpu().numpy()
+    on = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens, x_dtype=dtype, mx_scaled_mfma=True)
+    off = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens, x_dtype=dtype)
+    # the switch took: every projection with MXFP4 experts is on the block-scaled kernel, none without the switch
+    assert on.mx_scaled_slots() == sum(1 << s for s in range(3) if "MXFP4" in formats[s]) and off.mx_scaled_slots() == 0
+    scaled = on.run(*args).cpu().numpy()
+    plain = off.run(*args).cpu().numpy()
     err_scaled, err_plain = rel_l2(scaled, expect), rel_l2(plain, expect)
     print(f"MXFP4 prefill {case}: block-scaled MFMA {err_scaled:.3e}, fp16 tiles {err_plain:.3e}")
     assert np.isfinite(scaled).all()

@@ -488,3 +488,35 @@ def test_relu_squared_activation_against_exact_arithmetic():
     assert got[up < 0].view(np.uint16).max() == 0
     assert np.isinf(got[up == np.float16(300.0)][0])
     assert np.all(got[~finite].view(np.uint16) == 0)
+
+
+def test_shared_expert_epilogue_special_cases():
+    """O.shared_expert_epilogue (mfq/kernels/cuda/mfe_ffn_device.cuh:1249-1263) pinned by what its four operations fix:
+    a gate of 0 leaves the fp16-rounded routed sum, a gate of 1 adds the shared row as it is, a shared row of zeros adds
+    nothing, the routed sum is rounded to fp16 before the add (a value between two halves moves), and with fp16 gate
+    values the product is rounded to fp16 before the add (shared_product_half) while with fp32 gates it is not."""
+    routed = np.array([[1.0, 1.0 + 2.0 ** -12, 1000.25, -3.0e-5]], dtype=np.float32)
+    shared = np.array([[0.5, -2.0, 3.0, 1.0]], dtype=np.float16)
+    rounded = routed.astype(np.float16).astype(np.float32)
+    assert rounded[0, 1] != routed[0, 1] and rounded[0, 2] != routed[0, 2]          # the cases do exercise the rounding
+    zero_gate = O.shared_expert_epilogue(routed, shared, np.array([0.0], dtype=np.float32))
+    assert np.array_equal(zero_gate.view(np.uint32), rounded.view(np.uint32))
+    one_gate = O.shared_expert_epilogue(routed, shared, np.array([1.0], dtype=np.float32))
+    assert np.array_equal(one_gate, rounded + shared.astype(np.float32))
+    no_shared = O.shared_expert_epilogue(routed, np.zeros_like(shared), np.array([0.7], dtype=np.float32))
+    assert np.array_equal(no_shared.view(np.uint32), rounded.view(np.uint32))
+    # product rounding: 0.3 (fp16 0.30004883) * 3.0 = 0.90014648..., not a half
+    gate16 = np.array([0.3], dtype=np.float16)
+    exact = float(gate16[0]) * 3.0
+    as_half = float(np.float16(exact))
+    assert as_half != np.float32(exact)
+    half_product = O.shared_expert_epilogue(np.zeros((1, 4), np.float32), shared, gate16)
+    float_product = O.shared_expert_epilogue(np.zeros((1, 4), np.float32), shared, gate16.astype(np.float32))
+    assert half_product[0, 2] == np.float32(as_half) and float_product[0, 2] == np.float32(exact)
+    # independent restatement in float64 (every intermediate is exact in double except the two stated roundings)
+    rng = np.random.default_rng(77)
+    r = rng.normal(0, 3, (5, 64)).astype(np.float32)
+    sh = rng.normal(0, 2, (5, 64)).astype(np.float16)
+    g = rng.uniform(0, 1, 5).astype(np.float32)
+    want = (r.astype(np.float16).astype(np.float64) + (sh.astype(np.float64) * g.astype(np.float64)[:, None]).astype(np.float32)).astype(np.float32)
+    assert np.array_equal(O.shared_expert_epilogue(r, sh, g), want)

@@ -41,8 +41,11 @@ def test_static_scratch_entry_point_matches_the_workspace_entry_point():
     tensors, _ = synth.build_layer("test/static", experts, hidden, inter, mix=mix, mode="random")
     gate = R.MixedMoeRuntime(tensors[0])
     oracle = OracleMoeTensor(tensors[0])
-    # the larger call first (40 tokens: tile kernels), then smaller ones (decode kernels) that reuse the scratch
-    for tokens in (40, 7, 40, 1):
+    # the largest call first (512 tokens = 3072 pairs: the large plan kernel with its dynamic LDS and the tile kernels,
+    # near the top of what the static array holds), then smaller ones (40: the small plan and tile kernels, 7 and 1: the
+    # decode kernels) that reuse the scratch
+    assert 64 * 1024 < lib.mfq_amd_grouped_matmul_workspace(512, k, experts) <= lib.mfq_amd_grouped_matmul_static_capacity()
+    for tokens in (512, 40, 7, 40, 1):
         x = synth.to_bf16(synth.normal(f"test/static/x/{tokens}", (tokens, hidden)))
         ids = np.stack([np.random.default_rng(50 + t).permutation(experts)[:k] for t in range(tokens)]).astype(np.int32)
         ids[0, 0] = -1 if tokens > 1 else ids[0, 0]           # an unrouted pair
