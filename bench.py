@@ -86,8 +86,9 @@ def decode_workload(batch, steps, warmup, launch_mode, layers=2, batches=8, unif
                 layers=layers, batches=batches)
 
 
-def time_graph(step, steps, warmup):
-    """Eager warmup, then one HIP-graph replay of exactly `steps` steps between events."""
+def time_graph(step, steps, warmup, replays=7):
+    """Eager warmup, then HIP-graph replays of exactly `steps` steps between events: the median of `replays` replays
+    (bench/hip_nint_bench.cpp:58-86 takes the median of timed graph replays the same way)."""
     import torch
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -100,19 +101,25 @@ def time_graph(step, steps, warmup):
                 step(warmup + i)
         graph.replay()                      # first replay pays graph upload; not timed
         stream.synchronize()
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        start.record(stream)
-        graph.replay()
-        stop.record(stream)
-        stream.synchronize()
+        times = []
+        for _ in range(replays):
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(stream)
+            graph.replay()
+            stop.record(stream)
+            stream.synchronize()
+            times.append(start.elapsed_time(stop) / steps)
         torch.cuda.synchronize()
-    return start.elapsed_time(stop) / steps     # ms per step
+    times.sort()
+    return times[len(times) // 2]     # ms per step
 
 
 def stage_profile(work, steps):
     """Eager, instrumented pass: HIP events recorded by the library on the launch stream around each
-    stage; returns mean stage times (ms) and mean touched packed bytes per stage of a step."""
+    stage; returns mean stage times (ms) and mean touched packed bytes per stage of a step.  "empty_bracket" is what
+    two events recorded back to back read in the same run (the SwiGLU stage of a small batch, whose work runs inside the
+    down blocks, reads about that and nothing else); a bracket around one kernel reads the kernel plus half of it."""
     import numpy as np
     import torch
     for f in work["ffns"]:
@@ -122,6 +129,7 @@ def stage_profile(work, steps):
         work["step"](i)
         f = work["ffns"][i % work["layers"]]
         times = f.stage_times()
+        times["empty_bracket"] = f.empty_bracket_ms()
         for k, v in times.items():
             sums[k] = sums.get(k, 0.0) + v
         nbytes, n = f.touched_bytes()
@@ -200,11 +208,28 @@ def cpu_baseline(work, samples=7, budget_s=25.0):
         return float(np.median(times)), len(times)
 
     all_s, all_n = timed(True, budget_s * 0.4)
-    one_s, one_n = timed(False, budget_s * 0.6)
+    one_s, one_n = timed(False, budget_s * 0.5)
     cores = int(ref.ref_pool_participants())
+    # the hot variant of bench/cpu_nvq_bench.cpp:79-119: a working set that stays in the last-level cache (the ten
+    # experts of token 0, about 17 MB of packed weights, called again and again); the batch-16 layer above is the
+    # rotating one (about 237 MB of packed weights per call: every call streams its experts from memory)
+    hot_experts = {e: [0] for e, toks in by_expert.items() if 0 in toks}
+    hot = O.RefLayer({e: layouts[e] for e in hot_experts}, hot_experts, x)
+
+    def timed_hot(pooled):
+        hot.run(pooled)
+        times = []
+        for _ in range(samples):
+            t0 = time.perf_counter(); hot.run(pooled); times.append(time.perf_counter() - t0)
+        return float(np.median(times))
+
+    hot_all, hot_one = timed_hot(True), timed_hot(False)
     return {"value": tokens / all_s, "unit": "tok/s", "cores": cores, "kind": "reference", "samples": all_n,
-            "ms_per_layer": all_s * 1e3,
+            "ms_per_layer": all_s * 1e3, "working_set": "rotating: every call streams the routed experts of the batch from memory",
             "one_thread": {"value": tokens / one_s, "unit": "tok/s", "cores": 1, "samples": one_n, "ms_per_layer": one_s * 1e3},
+            "hot": {"sample": f"token 0 alone ({len(hot_experts)} experts, working set inside the last-level cache), median of {samples}",
+                    "value": 1.0 / hot_all, "unit": "tok/s", "cores": cores, "ms_per_layer": hot_all * 1e3,
+                    "one_thread": {"value": 1.0 / hot_one, "unit": "tok/s", "cores": 1, "ms_per_layer": hot_one * 1e3}},
             "sample": sample + "; NINT and NVQ rows through the reference library (all cores: its pinned expert pool), MXFP4 rows and "
                                "the SwiGLU chain through the C restatement; median"}
 
@@ -343,8 +368,14 @@ def main():
         g, d, _ = stage_bytes(work, i)
         gu_bytes += g / n
         dn_bytes += d / n
-    gu_gbs = gu_bytes / (stages["gate_up"] / 1e3) / 1e9
-    dn_gbs = dn_bytes / (stages["down"] / 1e3) / 1e9
+    # Two events recorded back to back read `empty` (about 4.5 us: two event packets); a bracket around one kernel holds
+    # the kernel and one of the two, so kernel time = bracket - empty / 2.  The kernel trace of the same command
+    # (profiles/) agrees with this form: 37.25 us traced against 39.56 - 4.53 / 2 = 37.3 us for the gate+up launch,
+    # 24.6 against 26.86 - 2.27 = 24.6 us for the down launch.
+    empty = stages.get("empty_bracket", 0.0)
+    gu_ms, dn_ms = max(stages["gate_up"] - empty / 2, 1e-6), max(stages["down"] - empty / 2, 1e-6)
+    gu_gbs = gu_bytes / (gu_ms / 1e3) / 1e9
+    dn_gbs = dn_bytes / (dn_ms / 1e3) / 1e9
     layer_gbs = touched / (ms / 1e3) / 1e9
 
     result = {
@@ -358,19 +389,23 @@ def main():
                    "batch": args.batch, "experts": EXPERTS, "hidden": HIDDEN, "intermediate": INTER, "top_k": TOP_K,
                    "format_mix": "NINT2 .10 NINT3 .25 NINT4 .30 NINT8 .05 NVQ3J-L .20 MXFP4 .10",
                    "rotation": f"{work['batches']} token batches x {work['layers']} layer copies",
-                   "launch_mode": args.launch_mode, "timing": "HIP-graph replay of the K steps"},
+                   "launch_mode": args.launch_mode, "timing": "median of 7 HIP-graph replays of the K steps"},
         "packed_weight_GBps": layer_gbs, "packed_weight_frac_hbm": layer_gbs / HBM_PEAK_GBS,
         "touched_bytes_per_step": touched, "distinct_experts_per_step": distinct,
-        "roofline": {"bound": "hbm", "kernel": "moe_rows_fast_kernel<64, true, 16> (gate+up stage)", "achieved": gu_gbs,
+        "roofline": {"bound": "hbm", "kernel": "moe_rows_fast_kernel<64, 1, 16> (gate+up stage)", "achieved": gu_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gu_gbs / HBM_PEAK_GBS,
                      "traffic": measured_traffic(args.batch),
                      "traffic_source": "profiles/moe_rows_fast_cfg4_b16_pmc.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, "
                                        "not read in this run)",
-                     "bytes_per_launch": gu_bytes, "ms_per_launch": stages["gate_up"],
+                     "bytes_per_launch": gu_bytes, "ms_per_launch": gu_ms, "ms_bracket": stages["gate_up"], "ms_empty_bracket": empty,
                      "method": "HIP events recorded by the library on the launch stream around each stage, eager pass "
-                               "of the same steps after the timed graph replay",
-                     "down_stage": {"achieved": dn_gbs, "frac": dn_gbs / HBM_PEAK_GBS, "bytes_per_launch": dn_bytes,
-                                    "ms_per_launch": stages["down"]},
+                               "of the same steps after the timed graph replays; two events back to back read "
+                               "ms_empty_bracket (measured behind the last stage of every step), a bracket around one kernel holds "
+                               "the kernel and one of the two event packets, so ms_per_launch = ms_bracket - ms_empty_bracket / 2; "
+                               "profiles/ holds the kernel trace of the same command, which agrees with this form",
+                     "down_stage": {"kernel": "moe_rows_fast_kernel<16, 2, 16> (down stage, SwiGLU inside)", "achieved": dn_gbs,
+                                    "frac": dn_gbs / HBM_PEAK_GBS, "bytes_per_launch": dn_bytes,
+                                    "ms_per_launch": dn_ms, "ms_bracket": stages["down"]},
                      "stages_ms": stages},
     }
     if not args.no_cpu:
@@ -379,7 +414,7 @@ def main():
         result["cpu_baseline"] = None
     if not args.no_extra:
         extra = {}
-        for b in (1, 4):
+        for b in (1, 2, 4, 8):
             w = decode_workload(b, args.steps, args.warmup, args.launch_mode)
             m = time_graph(w["step"], args.steps, args.warmup)
             st, tb, dx = stage_profile(w, min(args.steps, 16))

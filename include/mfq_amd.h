@@ -262,6 +262,10 @@ int mfq_amd_moe_ffn_touched_bytes(mfq_amd_moe_ffn* ffn, int64_t* bytes, int32_t*
  * which times stages with CudaProfiler::measure (ops/include/cuda_execution.h:109-150). */
 int mfq_amd_moe_ffn_enable_timing(mfq_amd_moe_ffn* ffn, int32_t enable);
 int mfq_amd_moe_ffn_stage_times(mfq_amd_moe_ffn* ffn, float* ms5);
+/* What a stage bracket reads when nothing is launched inside it: the elapsed time between two events recorded back to
+ * back behind the last stage of the same run (a few microseconds on this part).  Stage times of short kernels are read
+ * net of it. */
+int mfq_amd_moe_ffn_empty_bracket_ms(mfq_amd_moe_ffn* ffn, float* ms);
 void mfq_amd_moe_ffn_destroy(mfq_amd_moe_ffn* ffn);
 
 /* One mixed-format projection for routed pairs: out_dev f16 [tokens, k, out_per_expert].

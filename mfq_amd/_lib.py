@@ -93,6 +93,7 @@ EXPORTS = {
     "mfq_amd_moe_ffn_touched_bytes": (C.c_int, [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int32)]),
     "mfq_amd_moe_ffn_enable_timing": (C.c_int, [C.c_void_p, C.c_int32]),
     "mfq_amd_moe_ffn_stage_times": (C.c_int, [C.c_void_p, C.POINTER(C.c_float)]),
+    "mfq_amd_moe_ffn_empty_bracket_ms": (C.c_int, [C.c_void_p, C.POINTER(C.c_float)]),
     "mfq_amd_moe_ffn_destroy": (None, [C.c_void_p]),
     "mfq_amd_grouped_matmul_workspace": (C.c_int64, [C.c_int32, C.c_int32, C.c_int32]),
     "mfq_amd_grouped_matmul": (C.c_int, [C.POINTER(MoeTensor), C.c_void_p, C.c_int32, C.c_int32, C.c_void_p,

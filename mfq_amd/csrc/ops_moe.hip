@@ -678,7 +678,7 @@ struct mfq_amd_moe_ffn {
     uint16_t* d_shared_out = nullptr;
     bool decode_needs_items = true;   // some decode work runs on the exact kernels, which read the item lists
     bool timing = false;
-    hipEvent_t events[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    hipEvent_t events[7] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};   // the last closes an empty bracket
 
     ~mfq_amd_moe_ffn() {
         void* all[] = {d_pools, d_pool_class, d_pool_bytes, d_expert_pool, d_expert_info, d_expert_words, d_item_info, d_pair_items, d_items, d_class_offsets, d_tile_items,
@@ -1024,7 +1024,7 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
 
         // (a layer with a shared expert sums the pair rows in its own epilogue)
         if (reduce) launch_weighted_reduce(f->d_pairs, route_weights_dev, ids_dev, E, tokens, k, H, out_dev, f->config.out_dtype, stream);
-        f->mark(5, stream);
+        f->mark(5, stream); f->mark(6, stream);
     }
 }
 }  // namespace
@@ -1169,6 +1169,15 @@ extern "C" int mfq_amd_moe_ffn_stage_times(mfq_amd_moe_ffn* f, float* ms5) {
         MFQ_REQUIRE(f->timing && f->events[0], "stage timing is not enabled");
         MFQ_HIP(hipEventSynchronize(f->events[5]));
         for (int i = 0; i < 5; ++i) MFQ_HIP(hipEventElapsedTime(&ms5[i], f->events[i], f->events[i + 1]));
+    });
+}
+
+extern "C" int mfq_amd_moe_ffn_empty_bracket_ms(mfq_amd_moe_ffn* f, float* ms) {
+    return guarded([&] {
+        MFQ_REQUIRE(f && ms, "null argument");
+        MFQ_REQUIRE(f->timing && f->events[0], "stage timing is not enabled");
+        MFQ_HIP(hipEventSynchronize(f->events[6]));
+        MFQ_HIP(hipEventElapsedTime(ms, f->events[5], f->events[6]));
     });
 }
 

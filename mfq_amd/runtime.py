@@ -348,6 +348,12 @@ class MfeFfnRuntime:
         L.check(L.lib().mfq_amd_moe_ffn_stage_times(self._handle, ms))
         return dict(zip(("plan", "gate_up", "swiglu", "down", "reduce"), (float(v) for v in ms)))
 
+    def empty_bracket_ms(self) -> float:
+        """Milliseconds between two events recorded back to back behind the last stage of the last run."""
+        ms = C.c_float(0.0)
+        L.check(L.lib().mfq_amd_moe_ffn_empty_bracket_ms(self._handle, C.byref(ms)))
+        return float(ms.value)
+
     def touched_bytes(self) -> tuple[int, int]:
         nbytes, distinct = C.c_int64(), C.c_int32()
         L.check(L.lib().mfq_amd_moe_ffn_touched_bytes(self._handle, C.byref(nbytes), C.byref(distinct)))
