@@ -205,7 +205,12 @@ typedef struct mfq_amd_moe_ffn_config {
     int32_t expert_activation; /* 0: hidden = silu(gate) * up; 1: hidden = relu(up)^2 and no gate projection: gate.pool_count
                                   must be 0 and swiglu_limit 0 (MfeFfnBatch::expert_activation, mfq/kernels/cuda/mfe_ffn.h:79-82,
                                   :107-110) */
-    int32_t reserved[1];
+    int32_t group_pairs;       /* decode: 1 = a block of the rows kernels serves up to four pairs that are routed to the same
+                                  expert (the expert's rows are fetched and decoded once for the group: the per-token-group
+                                  form of mfq/kernels/cuda/mfe_mxfp4_dot.cuh:36-68, mfe_ffn_device.cuh:916-1006); 0 = one pair
+                                  per block, pairs of one expert next to each other so that its rows leave HBM once (the
+                                  default: it measured faster at every batch and expert count tried, the groups' blocks hold
+                                  twice the registers and half the waves) */
 } mfq_amd_moe_ffn_config;
 
 /* create may allocate and synchronise; run allocates nothing, does not synchronise and can be

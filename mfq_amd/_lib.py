@@ -48,7 +48,7 @@ class MoeFfnConfig(C.Structure):
                 ("top_k", C.c_int32), ("max_tokens", C.c_int32), ("x_dtype", C.c_int32),
                 ("out_dtype", C.c_int32), ("swiglu_limit", C.c_float), ("decode_token_limit", C.c_int32),
                 ("launch_mode", C.c_int32), ("mx_scaled_mfma", C.c_int32), ("expert_activation", C.c_int32),
-                ("reserved", C.c_int32 * 1)]
+                ("group_pairs", C.c_int32)]
 
 
 EXPORTS = {

@@ -50,6 +50,8 @@ struct RowsArgs {
     int32_t rows_per_block;            // streaming kernel: output rows per block, a multiple of rows_fast_min_block()
     int32_t exact_only;                // exact kernel: 1 = only items whose pool is marked kPoolExactOnly
     int32_t tile_slots;                // streaming tile kernel: slots of the launch (set by its launcher)
+    int32_t grouped;                   // streaming rows kernel: pair_items carry group sizes (PlanExtras::group_pairs): a block
+                                       // per group of up to kGroupPairs pairs of one expert
 };
 
 // True when the streaming fast path serves rows of this width and activation type.

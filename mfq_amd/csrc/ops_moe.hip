@@ -140,61 +140,76 @@ __device__ __forceinline__ void hidden_to_lds(const RowsArgs& a, int pair, Hidde
 // One block = one routed pair x rows_per_block output rows of its expert; a quarter of the rows per
 // wave.  Pairs of one expert sit next to each other in the grid, and the same row tile of
 // neighbouring pairs lands on the same XCD, so an expert's weights come from HBM once.
-template <int CLS, int LPR, int XMODE, int SLOTS, int IB>
+// NT > 1: the block multiplies the rows with the activations of up to NT pairs that the plan grouped because they are
+// routed to the same expert (PairItem::cls carries their number above bit 16): the packed rows are fetched and decoded
+// once for the group.  `pairs[n]` for n >= count repeat the first pair and store nothing.
+template <int CLS, int LPR, int XMODE, int SLOTS, int IB, int NT>
 __device__ __forceinline__ void rows_fast_pair(const RowsArgs& a, const mfq_amd_projection& pool, const PairItem& item, int slot,
-                                               unsigned char* lds, HiddenLds* hidden) {
+                                               unsigned char* lds, HiddenLds* hidden, const int (&pairs)[NT], int count) {
     const FastCtx<CLS> ctx = fast_ctx<CLS>(pool, item.local, lds);
     const int wave = uniform(static_cast<int>(threadIdx.x / kWave));
     const int rows_per_wave = a.rows_per_block / 4;
     const int row_begin = blockIdx.x * a.rows_per_block + wave * rows_per_wave;
-    const int pair = item.pair;
-    // the hidden row of the pair: computed while the first packed rows are on their way
+    // the hidden rows of the pairs: computed while the first packed rows are on their way
     auto prologue = [&] {
         if constexpr (XMODE == kXScaled) {
-            hidden_to_lds(a, pair, hidden);
-            if (threadIdx.x == 0) {
+#pragma unroll
+            for (int n = 0; n < NT; ++n) {
+                if (n > 0 && n >= count) break;           // uniform over the block: every thread takes the same turns
+                hidden_to_lds(a, pairs[n], &hidden[n]);
+            }
+            if (threadIdx.x < NT && static_cast<int>(threadIdx.x) < (count > 1 ? count : 1)) {
+                HiddenLds* h = &hidden[threadIdx.x];
                 float down, up;
-                uint32_t largest = hidden->wave_largest[0];
-                for (int w = 1; w < 4; ++w) largest = hidden->wave_largest[w] > largest ? hidden->wave_largest[w] : largest;
+                uint32_t largest = h->wave_largest[0];
+                for (int w = 1; w < 4; ++w) largest = h->wave_largest[w] > largest ? h->wave_largest[w] : largest;
                 normaliser(half_bits_to_float(static_cast<uint16_t>(largest)), down, up);
-                hidden->scale[0] = down; hidden->scale[1] = up;
+                h->scale[0] = down; h->scale[1] = up;
             }
             __syncthreads();
         }
     };
     if (row_begin >= a.out_rows) { prologue(); return; }
     const int row_end = row_begin + rows_per_wave < a.out_rows ? row_begin + rows_per_wave : a.out_rows;
-    uint16_t* out = a.out + (slot - a.slot_base) * a.out_slot_stride + pair * a.out_pair_stride;
-    const int64_t source = a.in_per_pair ? pair : pair / a.top_k;
-    const XSource xs[1] = {{XMODE == kXPacked ? static_cast<const void*>(a.in_packed + source * a.in_packed_stride)
-                            : XMODE == kXScaled ? static_cast<const void*>(hidden->values) : pair_source(a, pair),
-                            XMODE == kXScaled ? MFQ_AMD_F16 : a.in_dtype, XMODE == kXScaled ? true : a.in_vector_ok != 0,
-                            hidden->scale}};
+    uint16_t* outs[NT];
+    XSource xs[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+        const int pair = pairs[n];
+        const int staged = n < count ? n : 0;
+        outs[n] = a.out + (slot - a.slot_base) * a.out_slot_stride + pair * a.out_pair_stride;
+        const int64_t source = a.in_per_pair ? pair : pair / a.top_k;
+        xs[n] = XSource{XMODE == kXPacked ? static_cast<const void*>(a.in_packed + source * a.in_packed_stride)
+                        : XMODE == kXScaled ? static_cast<const void*>(hidden[staged].values) : pair_source(a, pair),
+                        XMODE == kXScaled ? MFQ_AMD_F16 : a.in_dtype, XMODE == kXScaled ? true : a.in_vector_ok != 0,
+                        hidden[staged].scale};
+    }
     constexpr int kRing = FastClass<CLS>::kRing < SLOTS || SLOTS == 0 ? FastClass<CLS>::kRing : SLOTS;
-    auto store = [&](int, int row, float value) { out[row] = float_to_half_bits(value); };
+    auto store = [&](int n, int row, float value) { if (NT == 1 || n < count) outs[n][row] = float_to_half_bits(value); };
     if constexpr (FastClass<CLS>::kNint && SLOTS > 0) {
         // straight-line variants: the levels of a row slot as shared level words where the row's geometry allows
         if (nint_level_words_cover(ctx.groups, nint_level_word_stride(FastClass<CLS>::kGs), 32 / (kWave / LPR))) {
-            fast_rows<CLS, LPR, 1, 1, kRing, XMODE, SLOTS, IB, true>(ctx, xs, a.in_width, row_begin, row_end, a.out_rows, store, prologue);
+            fast_rows<CLS, LPR, 1, NT, kRing, XMODE, SLOTS, IB, true>(ctx, xs, a.in_width, row_begin, row_end, a.out_rows, store, prologue);
             return;
         }
     }
-    fast_rows<CLS, LPR, 1, 1, kRing, XMODE, SLOTS, IB>(ctx, xs, a.in_width, row_begin, row_end, a.out_rows, store, prologue);
+    fast_rows<CLS, LPR, 1, NT, kRing, XMODE, SLOTS, IB>(ctx, xs, a.in_width, row_begin, row_end, a.out_rows, store, prologue);
 }
 
-template <int CLS, int LPR, int XMODE, int SLOTS>
-__device__ __forceinline__ void rows_fast_block(const RowsArgs& a, const PairItem& item, int slot, unsigned char* lds, HiddenLds* hidden) {
+template <int CLS, int LPR, int XMODE, int SLOTS, int NT>
+__device__ __forceinline__ void rows_fast_block(const RowsArgs& a, const PairItem& item, int slot, unsigned char* lds, HiddenLds* hidden,
+                                                const int (&pairs)[NT], int count) {
     const mfq_amd_projection& pool = a.pools[item.pool];
     if constexpr (FastClass<CLS>::kNvq) {
         nvq_fast_tables(pool, lds);
         __syncthreads();
         // the index width of the format fixes the bit positions of every index: one copy of the row loop each
         const int index_bits = nvq_format_index_bits(pool.format);
-        if (index_bits == 10) rows_fast_pair<CLS, LPR, XMODE, SLOTS, 10>(a, pool, item, slot, lds, hidden);
-        else if (index_bits == 9) rows_fast_pair<CLS, LPR, XMODE, SLOTS, 9>(a, pool, item, slot, lds, hidden);
-        else rows_fast_pair<CLS, LPR, XMODE, SLOTS, 8>(a, pool, item, slot, lds, hidden);
+        if (index_bits == 10) rows_fast_pair<CLS, LPR, XMODE, SLOTS, 10, NT>(a, pool, item, slot, lds, hidden, pairs, count);
+        else if (index_bits == 9) rows_fast_pair<CLS, LPR, XMODE, SLOTS, 9, NT>(a, pool, item, slot, lds, hidden, pairs, count);
+        else rows_fast_pair<CLS, LPR, XMODE, SLOTS, 8, NT>(a, pool, item, slot, lds, hidden, pairs, count);
     } else {
-        rows_fast_pair<CLS, LPR, XMODE, SLOTS, 0>(a, pool, item, slot, lds, hidden);
+        rows_fast_pair<CLS, LPR, XMODE, SLOTS, 0, NT>(a, pool, item, slot, lds, hidden, pairs, count);
     }
 }
 
@@ -204,22 +219,36 @@ __device__ __forceinline__ void rows_fast_block(const RowsArgs& a, const PairIte
 // covers 4 * SLOTS * (64 / LPR) rows; 0 = taken from rows_per_block at run time.
 // XMODE: kXRaw / kXPacked: activations from RowsArgs::in / in_packed; kXScaled: the block computes the hidden row of
 // its pair from RowsArgs::gu first (down projection of the FFN; rows of at most 512 columns).
-template <int LPR, int XMODE, int SLOTS>
+// NT: 1: a block per pair.  kGroupPairs: the plan has grouped up to that many neighbouring pairs of one expert; the
+// block of a group's first pair multiplies for all of them and the blocks of the others return at once.
+template <int LPR, int XMODE, int SLOTS, int NT>
 __global__ void __launch_bounds__(256) moe_rows_fast_kernel(RowsArgs a) {
     // The NVQ tables sit in statically sized LDS: their addresses are then constants of the instruction
     // stream.  Four blocks of a CU hold 4 x 35 KB of the 160 KB, which the register budget allows anyway.
     __shared__ __attribute__((aligned(16))) unsigned char lds[kNvqFastLdsBytes];
-    __shared__ __attribute__((aligned(16))) HiddenLds hidden[1];
+    __shared__ __attribute__((aligned(16))) HiddenLds hidden[NT];
     const int slot = a.slot_base + blockIdx.z;
-    const PairItem item = a.pair_items[static_cast<int64_t>(slot) * a.pairs + blockIdx.y];
+    const PairItem* list = a.pair_items + static_cast<int64_t>(slot) * a.pairs;
+    PairItem item = list[blockIdx.y];
+    int pairs[NT];
+    int count = 1;
+    pairs[0] = item.pair;
+    if constexpr (NT > 1) {
+        if (item.cls < 0) return;
+        count = item.cls >> kGroupCountShift;
+        item.cls &= (1 << kGroupCountShift) - 1;
+        if (count == 0) return;                           // a pair that the block of its group's first pair serves
+#pragma unroll
+        for (int n = 1; n < NT; ++n) pairs[n] = n < count ? list[blockIdx.y + n].pair : item.pair;
+    }
     switch (item.cls) {
-        case K_NINT_2_16: rows_fast_block<K_NINT_2_16, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
-        case K_NINT_3_24: rows_fast_block<K_NINT_3_24, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
-        case K_NINT_4_24: rows_fast_block<K_NINT_4_24, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
-        case K_NINT_4_32: rows_fast_block<K_NINT_4_32, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
-        case K_NINT_8_48: rows_fast_block<K_NINT_8_48, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
-        case K_NVQ_D4: rows_fast_block<K_NVQ_D4, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
-        case K_MXFP4: rows_fast_block<K_MXFP4, LPR, XMODE, SLOTS>(a, item, slot, lds, hidden); break;
+        case K_NINT_2_16: rows_fast_block<K_NINT_2_16, LPR, XMODE, SLOTS, NT>(a, item, slot, lds, hidden, pairs, count); break;
+        case K_NINT_3_24: rows_fast_block<K_NINT_3_24, LPR, XMODE, SLOTS, NT>(a, item, slot, lds, hidden, pairs, count); break;
+        case K_NINT_4_24: rows_fast_block<K_NINT_4_24, LPR, XMODE, SLOTS, NT>(a, item, slot, lds, hidden, pairs, count); break;
+        case K_NINT_4_32: rows_fast_block<K_NINT_4_32, LPR, XMODE, SLOTS, NT>(a, item, slot, lds, hidden, pairs, count); break;
+        case K_NINT_8_48: rows_fast_block<K_NINT_8_48, LPR, XMODE, SLOTS, NT>(a, item, slot, lds, hidden, pairs, count); break;
+        case K_NVQ_D4: rows_fast_block<K_NVQ_D4, LPR, XMODE, SLOTS, NT>(a, item, slot, lds, hidden, pairs, count); break;
+        case K_MXFP4: rows_fast_block<K_MXFP4, LPR, XMODE, SLOTS, NT>(a, item, slot, lds, hidden, pairs, count); break;
         default: break;   // unrouted, exact-only pools and classes without a fast path
     }
 }
@@ -461,28 +490,31 @@ void launch_rows_fast(const RowsArgs& args, int slots, bool nvq, hipStream_t str
     const bool narrow = args.in_width <= 16 * dev::kLaneColumns;
     const int wave_slots = args.rows_per_block / (narrow ? 16 : 4);
     auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(256), bytes, stream, args); };
+    // by the number of row slots per wave: straight-line variants for the block heights the FFN uses, the looped kernel
+    // (0) for the rest; by the activations: hidden rows computed by the block, rows in the packed form, plain rows
+    auto by_slots = [&](auto lpr, auto xmode, auto nt) {
+        constexpr int L = decltype(lpr)::value, X = decltype(xmode)::value, N = decltype(nt)::value;
+        if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<L, X, 4, N>);
+        else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<L, X, 8, N>);
+        else if (wave_slots == 16) launch(dev::moe_rows_fast_kernel<L, X, 16, N>);
+        else launch(dev::moe_rows_fast_kernel<L, X, 0, N>);
+    };
+    auto by_group = [&](auto lpr, auto xmode) {
+        if (args.grouped) by_slots(lpr, xmode, std::integral_constant<int, kGroupPairs>{});
+        else by_slots(lpr, xmode, std::integral_constant<int, 1>{});
+    };
+    using lanes16 = std::integral_constant<int, 16>;
+    using lanes64 = std::integral_constant<int, 64>;
     if (args.gu != nullptr) {
         MFQ_REQUIRE(narrow && args.in_per_pair && args.sigmoid != nullptr, "the fused SwiGLU serves rows of at most 512 columns");
-        if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 4>);
-        else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 8>);
-        else if (wave_slots == 16) launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 16>);
-        else launch(dev::moe_rows_fast_kernel<16, dev::kXScaled, 0>);
+        by_group(lanes16{}, std::integral_constant<int, dev::kXScaled>{});
     } else if (args.in_packed != nullptr) {
-        // straight-line variants for the block heights the FFN uses, the looped kernel for the rest
-        if (narrow) {
-            if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 4>);
-            else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 8>);
-            else if (wave_slots == 16) launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 16>);
-            else launch(dev::moe_rows_fast_kernel<16, dev::kXPacked, 0>);
-        } else {
-            if (wave_slots == 4) launch(dev::moe_rows_fast_kernel<64, dev::kXPacked, 4>);
-            else if (wave_slots == 8) launch(dev::moe_rows_fast_kernel<64, dev::kXPacked, 8>);
-            else if (wave_slots == 16) launch(dev::moe_rows_fast_kernel<64, dev::kXPacked, 16>);
-            else launch(dev::moe_rows_fast_kernel<64, dev::kXPacked, 0>);
-        }
+        if (narrow) by_group(lanes16{}, std::integral_constant<int, dev::kXPacked>{});
+        else by_group(lanes64{}, std::integral_constant<int, dev::kXPacked>{});
     } else {
-        if (narrow) launch(dev::moe_rows_fast_kernel<16, dev::kXRaw, 0>);
-        else launch(dev::moe_rows_fast_kernel<64, dev::kXRaw, 0>);
+        MFQ_REQUIRE(!args.grouped, "grouped pairs are served from packed activations");
+        if (narrow) launch(dev::moe_rows_fast_kernel<16, dev::kXRaw, 0, 1>);
+        else launch(dev::moe_rows_fast_kernel<64, dev::kXRaw, 0, 1>);
     }
     check_launch("moe_rows_fast_kernel");
 }
@@ -706,6 +738,7 @@ extern "C" int mfq_amd_moe_ffn_create(const mfq_amd_moe_ffn_config* config, mfq_
         MFQ_REQUIRE(c.launch_mode == 0 || c.launch_mode == 1, "unknown launch mode");
         MFQ_REQUIRE(c.mx_scaled_mfma == 0 || c.mx_scaled_mfma == 1, "mx_scaled_mfma must be 0 or 1");
         MFQ_REQUIRE(c.expert_activation == 0 || c.expert_activation == 1, "expert_activation must be 0 or 1");
+        MFQ_REQUIRE(c.group_pairs == 0 || c.group_pairs == 1, "group_pairs must be 0 or 1");
         MFQ_REQUIRE(c.swiglu_limit >= 0.0f, "swiglu_limit must not be negative");
         const bool gated = c.expert_activation == 0;
         if (gated) {
@@ -878,6 +911,13 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         const bool fuse_swiglu = fast_mode && !f->decode_needs_items && I <= 16 * dev::kLaneColumns && rows_fast_geometry(I, MFQ_AMD_F16) &&
                                  (pairs <= kFusedSwigluPairs || (H + down_height - 1) / down_height <= kFusedSwigluBlocks);
         const bool pack_hidden = fast_mode && !fuse_swiglu && f->d_hidden_packed != nullptr;
+        // On request the plan groups up to kGroupPairs neighbouring pairs of one expert and a block of the rows kernels
+        // fetches and decodes the expert's rows once for the group (the reference's per-token-group form,
+        // mfq/kernels/cuda/mfe_mxfp4_dot.cuh:36-68).  Not the default: with the pairs of an expert next to each other its
+        // rows come out of the L2 for all but the first pair anyway, and the group's blocks hold twice the registers, so
+        // half the waves (2048 <-> 512 layer of 16..64 experts, top-8, batches 4..32: 38..130 us per step in groups
+        // against 28..90 us with a block per pair).
+        x.group_pairs = x.pairs_only && pack_x && (fuse_swiglu || pack_hidden) && f->config.group_pairs == 1;
         if (pack_x) {
             plan.pack.src = x_dev; plan.pack.dst = f->d_x_packed; plan.pack.stride = dev::xpack_row_dwords(H);
             plan.pack.rows = tokens; plan.pack.width = H; plan.pack.dtype = f->config.x_dtype;
@@ -906,6 +946,7 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         rows.class_offsets = f->d_class_offsets; rows.tile_items = f->d_tile_items; rows.tile_offsets = f->d_tile_offsets;
         rows.expert_bounds = f->d_bounds; rows.ids_dst = f->d_ids_dst;
         rows.experts = E; rows.top_k = k; rows.tile_capacity = f->tile_capacity;
+        rows.grouped = x.group_pairs;
 
         int present[dev::K_CLASS_COUNT], bound[dev::K_CLASS_COUNT];
         // classes to launch over slots [slot_lo, slot_hi): every present class, or only those with
@@ -936,7 +977,10 @@ void ffn_run(mfq_amd_moe_ffn* f, const void* x_dev, const int32_t* ids_dev, cons
         auto rows_per_block = [&](int out_rows, int slots) {
             const int least = rows_fast_min_block(rows_in_width);
             int height = rows_in_width > 16 * dev::kLaneColumns ? 64 : 256;
-            while (height > least && static_cast<int64_t>(pairs) * slots * ((out_rows + height - 1) / height) < 1024) height /= 2;
+            // blocks of the launch along the pair axis: the pairs, or about the groups where blocks serve groups of pairs
+            int64_t units = pairs;
+            if (rows.grouped) units = std::max<int64_t>(std::min<int64_t>(pairs, E), (pairs + kGroupPairs - 1) / kGroupPairs);
+            while (height > least && units * slots * ((out_rows + height - 1) / height) < 1024) height /= 2;
             return height;
         };
         auto run_rows = [&](int slot_lo, int slot_hi) {

@@ -1140,13 +1140,37 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_pairs_kernel(PlanArgs
             smaller += below(v0) + below(v1) + below(v2) + below(v3);
         }
         for (; q < end; q += 4) smaller += below(*reinterpret_cast<const uint4*>(&keys[s][q]));
+        // Groups: the pairs of one expert share the key's upper bits and sit next to each other in the order; a pair's
+        // place among them and their number are two more counts over the same keys (those below the expert's first
+        // possible key and those below the next expert's).  Every kGroupPairs-th pair of an expert opens a group.
+        int before_expert = 0, through_expert = 0;
+        if (x.group_pairs) {
+            const uint32_t first = mine & ~0x3ffu, next = first + 0x400u;
+            auto under = [](const uint4& v, uint32_t bound) { return (v.x < bound) + (v.y < bound) + (v.z < bound) + (v.w < bound); };
+            for (int g = begin; g < end; g += 4) {
+                const uint4 v = *reinterpret_cast<const uint4*>(&keys[s][g]);
+                before_expert += under(v, first);
+                through_expert += under(v, next);
+            }
+        }
         // the parts of an item sit in neighbouring lanes (2, 4 or 8 of them): data-parallel moves, no LDS round trip
-        if (parts > 1) smaller += __builtin_amdgcn_update_dpp(0, smaller, 0xB1, 0xF, 0xF, false);    // lane ^ 1
-        if (parts > 2) smaller += __builtin_amdgcn_update_dpp(0, smaller, 0x4E, 0xF, 0xF, false);    // lane ^ 2
-        if (parts > 4) smaller += __builtin_amdgcn_update_dpp(0, smaller, 0x141, 0xF, 0xF, false);   // the other quad of eight lanes
+        auto over_parts = [parts](int v) {
+            if (parts > 1) v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);    // lane ^ 1
+            if (parts > 2) v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);    // lane ^ 2
+            if (parts > 4) v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, false);   // the other quad of eight lanes
+            return v;
+        };
+        smaller = over_parts(smaller);
+        if (x.group_pairs) { before_expert = over_parts(before_expert); through_expert = over_parts(through_expert); }
         if (live && part == 0) {
             const int4 record = records[s][p];
-            x.pair_items[static_cast<int64_t>(s) * P + smaller] = PairItem{record.x, record.y, record.z, record.w};
+            int cls = record.w;
+            if (x.group_pairs && cls >= 0) {
+                const int place = smaller - before_expert, left = through_expert - smaller;      // left counts this pair
+                const int count = place % kGroupPairs == 0 ? (left < kGroupPairs ? left : kGroupPairs) : 0;
+                cls |= count << kGroupCountShift;
+            }
+            x.pair_items[static_cast<int64_t>(s) * P + smaller] = PairItem{record.x, record.y, record.z, cls};
         }
     }
 }

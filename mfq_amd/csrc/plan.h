@@ -33,8 +33,11 @@ struct PairItem {
     int32_t pair;     // index of the pair (token * top_k + route), -1 behind the last routed pair
     int32_t pool;     // index into the pool array
     int32_t local;    // index of the expert inside its pool
-    int32_t cls;      // kernel class (| kPoolExactOnly)
+    int32_t cls;      // kernel class (| kPoolExactOnly); with PlanExtras::group_pairs also, from bit kGroupCountShift, the
+                      // number of pairs of the group this pair opens (1..kGroupPairs), 0 for the other pairs of a group
 };
+constexpr int kGroupPairs = 4;          // pairs of one expert that one block of the streaming rows kernel serves together
+constexpr int kGroupCountShift = 16;
 
 // What the plan needs to know about one expert of one slot, resolved once when the pools are fixed.
 struct ExpertInfo {
@@ -80,6 +83,8 @@ struct PlanExtras {
     int32_t prefill_tile_m;
     int32_t want_tiles;                // 0: tile_items / tile_offsets are not needed (decode)
     int32_t want_items;                // 0: items / item_info / class_offsets are not needed (no exact-kernel work)
+    int32_t group_pairs;               // 1 (with pairs_only): neighbouring pairs of one expert form groups of up to kGroupPairs;
+                                       // PairItem::cls carries the group sizes
     int32_t pairs_only;                // 1 (at most kPlanSortPairs pairs, expert_info given, no want_items / want_tiles):
                                        // only pair_items is produced, by the kernel that ranks the pairs directly;
                                        // none of counts, expert_bounds, ids_dst, items, touched_bytes, distinct written

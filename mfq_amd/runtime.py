@@ -219,8 +219,9 @@ class MfeFfnRuntime:
     def __init__(self, gate: MixedMoeRuntime | None, up: MixedMoeRuntime, down: MixedMoeRuntime, top_k: int,
                  max_tokens: int, x_dtype: torch.dtype = torch.bfloat16, out_dtype: torch.dtype = torch.float32,
                  swiglu_limit: float = 0.0, decode_token_limit: int = 0, launch_mode: int = 0, mx_scaled_mfma: bool = False,
-                 expert_activation: int = 0):
-        """expert_activation 1: hidden = relu(up)^2, ``gate`` must be None (a relu-squared bank has no gate descriptor)."""
+                 expert_activation: int = 0, group_pairs: int = 0):
+        """expert_activation 1: hidden = relu(up)^2, ``gate`` must be None (a relu-squared bank has no gate descriptor).
+        group_pairs: 1 = decode blocks serve up to four pairs of one expert, 0 = one pair per block (faster as measured)."""
         if (gate is None) != (expert_activation == 1):
             raise ValueError("the gate projection is absent exactly when expert_activation is 1")
         self._keep = (gate, up, down)
@@ -239,6 +240,7 @@ class MfeFfnRuntime:
         config.decode_token_limit = decode_token_limit
         config.launch_mode = launch_mode
         config.mx_scaled_mfma = int(mx_scaled_mfma)
+        config.group_pairs = group_pairs
         handle = C.c_void_p()
         L.check(L.lib().mfq_amd_moe_ffn_create(C.byref(config), C.byref(handle)))
         self._handle = handle

@@ -55,6 +55,37 @@ def test_decode_ffn_vs_oracle(mode, tokens):
     assert nbytes > 0
 
 
+@pytest.mark.parametrize("tokens", [2, 5, 12, 16])
+def test_decode_blocks_that_serve_a_group_of_pairs_vs_oracle(tokens):
+    """Few experts, many pairs, group_pairs = 1: the plan groups up to four neighbouring pairs of one expert and one block
+    of the rows kernels multiplies for all of them (12 tokens x top-4 over 8 experts is six pairs per expert, i.e. groups
+    of four and two).  Against the oracle, and bit for bit against the same layer with one block per pair: a pair's
+    arithmetic does not depend on who shares its block."""
+    import torch
+    from mfq_amd import runtime as R
+    experts, hidden, inter, k = 8, 512, 128, 4
+    tensors, runtimes, _ = _layer("test/moe/groups", experts, hidden, inter, "random")
+    x, ids, weights = _inputs(f"test/moe/groups/in/{tokens}", tokens, experts, hidden, k)
+    if tokens >= 5:
+        ids = ids.copy(); ids[1, 2] = -1                           # an unrouted pair among the groups
+    args = (torch.from_numpy(x).to(torch.bfloat16).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(weights).cuda())
+    routed = ids >= 0
+    results = {}
+    for mode in (1, 0):
+        ffn = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=16, group_pairs=mode)
+        out = ffn.run(*args).cpu().numpy()
+        gu, pairs = ffn.stage_buffers(tokens)
+        results[mode] = (out, np.asarray(gu).reshape(tokens, k, -1)[routed], np.asarray(pairs).reshape(tokens, k, -1)[routed])
+    expect = oracle_layer(x, np.where(routed, ids, 0), np.where(routed, weights, 0.0).astype(np.float32), tensors)
+    for mode, (out, gu, pairs) in results.items():
+        err = rel_l2(out, expect)
+        print(f"grouped decode T={tokens} mode {mode}: rel-L2 {err:.3e}")
+        assert err <= FFN_TOL, mode
+        assert np.array_equal(gu.view(np.uint16), results[0][1].view(np.uint16)), mode
+        assert np.array_equal(pairs.view(np.uint16), results[0][2].view(np.uint16)), mode
+        assert np.array_equal(out.view(np.uint32), results[0][0].view(np.uint32)), mode
+
+
 def test_decode_stage_buffers_vs_oracle():
     """gate/up and per-pair down outputs, stage by stage."""
     import torch
