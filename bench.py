@@ -42,6 +42,8 @@ def parse_args():
     p.add_argument("--launch-mode", type=int, default=0)
     p.add_argument("--prefill-only", action="store_true",
                    help="run only the 4096-token prefill layer (a profiling aid: prints its own JSON line)")
+    p.add_argument("--prefill-mixed", action="store_true",
+                   help="with --prefill-only: the mixed-format layer alone, without the two all-MXFP4 layers")
     return p.parse_args()
 
 
@@ -351,6 +353,9 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+    if args.prefill_only and args.prefill_mixed:
+        print(json.dumps({"prefill_4096": prefill_measure()}))
+        return
     if args.prefill_only:
         print(json.dumps({"prefill_4096": prefill_measure(),
                           "prefill_4096_mxfp4_f16_tiles": prefill_measure(uniform="MXFP4"),

@@ -228,8 +228,11 @@ int mfq_amd_moe_ffn_run(mfq_amd_moe_ffn* ffn, const void* x_dev, const int32_t* 
  * copied, their device buffers stay borrowed.  run_shared is run() with the epilogue of mfe_ffn_down_reduce_kernel
  * (mfq/kernels/cuda/mfe_ffn_device.cuh:1249-1263): out = half(sum_r w * pair) + shared_ffn(x)[half] * shared_gate[token]
  * in fp32, written as config.out_dtype; shared_gate_dev holds one evaluated gate value per token (float32, float16 or
- * bfloat16; with float16 the product is rounded to fp16 first, the reference's shared_product_half).  Allocates
- * nothing, does not synchronise. */
+ * bfloat16; with float16 the product is rounded to fp16 first, the reference's shared_product_half).  The routed sum
+ * adds w * pair per route in route order with a separate multiply and add, which is what the oracle fixes; the
+ * reference's kernels write value += w * x (mfq/kernels/cuda/moe.cu:1511, mfe_ffn_device.cuh:1249-1263), which their
+ * compiler may contract to an FMA, so bit parity with them before the fp16 rounding is not pinned (no fixture of the
+ * reference covers it).  Allocates nothing, does not synchronise. */
 int mfq_amd_moe_ffn_set_shared(mfq_amd_moe_ffn* ffn, const mfq_amd_projection* gate, const mfq_amd_projection* up,
                                const mfq_amd_projection* down, int32_t shared_activation);
 int mfq_amd_moe_ffn_run_shared(mfq_amd_moe_ffn* ffn, const void* x_dev, const int32_t* ids_dev, const float* route_weights_dev,
