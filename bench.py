@@ -397,7 +397,7 @@ def main():
                    "launch_mode": args.launch_mode, "timing": "median of 7 HIP-graph replays of the K steps"},
         "packed_weight_GBps": layer_gbs, "packed_weight_frac_hbm": layer_gbs / HBM_PEAK_GBS,
         "touched_bytes_per_step": touched, "distinct_experts_per_step": distinct,
-        "roofline": {"bound": "hbm", "kernel": "moe_rows_fast_kernel<64, 1, 16> (gate+up stage)", "achieved": gu_gbs,
+        "roofline": {"bound": "hbm", "kernel": "moe_rows_fast_kernel<64, 1, 16, 1> (gate+up stage)", "achieved": gu_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gu_gbs / HBM_PEAK_GBS,
                      "traffic": measured_traffic(args.batch),
                      "traffic_source": "profiles/moe_rows_fast_cfg4_b16_pmc.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, "
@@ -408,7 +408,7 @@ def main():
                                "ms_empty_bracket (measured behind the last stage of every step), a bracket around one kernel holds "
                                "the kernel and one of the two event packets, so ms_per_launch = ms_bracket - ms_empty_bracket / 2; "
                                "profiles/ holds the kernel trace of the same command, which agrees with this form",
-                     "down_stage": {"kernel": "moe_rows_fast_kernel<16, 2, 16> (down stage, SwiGLU inside)", "achieved": dn_gbs,
+                     "down_stage": {"kernel": "moe_rows_fast_kernel<16, 2, 16, 1> (down stage, SwiGLU inside)", "achieved": dn_gbs,
                                     "frac": dn_gbs / HBM_PEAK_GBS, "bytes_per_launch": dn_bytes,
                                     "ms_per_launch": dn_ms, "ms_bracket": stages["down"]},
                      "stages_ms": stages},
