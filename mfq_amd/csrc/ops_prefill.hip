@@ -383,6 +383,58 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         states = state_word >> (state_bit & 7u);
     };
 
+    // Packed rows in coalesced runs (tiles of at most 64 pairs, classes whose lane blocks hold 16 bytes).  A weight load
+    // of the lane that will decode the data touches 32 rows x 32 bytes, and the address unit's time per load instruction
+    // follows the cache lines it touches, not the bytes it brings.  Here a wave loads the 64-byte runs that its 64 rows
+    // need for two steps with four lanes per row (16 rows per instruction: half the lines), parks them in a 4 KB
+    // piece of LDS of its own (the part of the activation buffers that tiles of this height leave unused) and reads them
+    // back in the layout of the MFMA operand, one 16-byte piece per lane, row and step.  Nothing is shared between
+    // waves, so no barrier is involved; the pieces of a row are swizzled so that neither the writes nor the reads meet
+    // in a bank.  The runs of the pair of steps after next are requested when those of the next pair have been read
+    // back, two steps before they are needed.
+    constexpr bool kStaged = PACKED && MT <= 2 && (CLS == K_NINT_4_24 || CLS == K_NINT_4_32 || CLS == K_MXFP4);
+    static_assert(!kStaged || 2 * 32 * 128 + 2 * 4096 <= kFastXBytes, "two waves park their runs behind the rows of a low tile");
+    u32x4 staged_rows[4] = {};
+    unsigned char* wave_stage = x_lds + (wave >> 1) * kFastXBytes + 2 * 32 * 128 + (wave & 1) * 4096;
+    auto stage_issue = [&](int pair_of_steps) {
+        const int last = steps / 2 - 1;
+        const int d = pair_of_steps < last ? pair_of_steps : last;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int row = row_block * kFastTileN + wave * 64 + 16 * i + (lane >> 2);
+            row = row < a.out_rows ? row : a.out_rows - 1;
+            const uint8_t* at = ctx.f0 + static_cast<uint32_t>(row) * static_cast<uint32_t>(ctx.row_bytes) +
+                                static_cast<uint32_t>((4 * d + (lane & 3)) * 16);
+            staged_rows[i] = *(const MFQ_GLOBAL u32x4_u*)at;
+        }
+    };
+    auto stage_swizzle = [](int row) { return (row >> 1) & 3; };
+    auto stage_commit = [&](FastRaw<CLS> (&even)[2], FastRaw<CLS> (&odd)[2]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 16 * i + (lane >> 2);
+            *reinterpret_cast<u32x4*>(wave_stage + r * 64 + (((lane & 3) ^ stage_swizzle(r)) << 4)) = staged_rows[i];
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int r = 32 * t + n;
+            const u32x4 first = *reinterpret_cast<const u32x4*>(wave_stage + r * 64 + ((h ^ stage_swizzle(r)) << 4));
+            const u32x4 second = *reinterpret_cast<const u32x4*>(wave_stage + r * 64 + (((2 + h) ^ stage_swizzle(r)) << 4));
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { even[t].q[k] = first[k]; odd[t].q[k] = second[k]; }
+        }
+    };
+    // MXFP4: the block scales still come one byte per lane, row and step
+    auto fetch_scales = [&](int step, FastRaw<CLS> (&raw)[2]) {
+        if constexpr (C::kMx) {
+            const int last = steps - 1;
+            const LaneBlock b = lane_block<C::kGs>(2 * (step < last ? step : last) + h, width, ctx.groups);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) raw[t].a = gload<uint8_t>(ctx.f1 + mx_fetch_at(rows[t], ctx.row_bytes, b).scale_byte);
+        }
+    };
+    constexpr int kScaleLoads = C::kMx ? 2 : 0;      // per call of fetch_scales
+
     float16_t acc[2][MT];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -391,19 +443,28 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[t][mt][i] = 0.0f;
 
-    FastRaw<CLS> ring[2][2];
+    FastRaw<CLS> ring[2][2] = {};
     u32x4 x_raw[4];
     if constexpr (PACKED) {
         x_direct(0);
     } else {
         x_load(0, x_raw);
     }
-    fetch(0, ring[0]);
-    fetch(1, ring[1]);
-    if constexpr (PACKED) {
-        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * 2 * fetch_loads<CLS>()) : "memory");   // the direct loads, not the weights
+    if constexpr (kStaged) {
+        stage_issue(0);
+        fetch_scales(0, ring[0]);
+        fetch_scales(1, ring[1]);
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(4 + 2 * kScaleLoads) : "memory");   // the direct loads, not the weights
+        stage_commit(ring[0], ring[1]);
+        stage_issue(1);
     } else {
-        x_store(0, x_raw);
+        fetch(0, ring[0]);
+        fetch(1, ring[1]);
+        if constexpr (PACKED) {
+            asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * 2 * fetch_loads<CLS>()) : "memory");   // the direct loads, not the weights
+        } else {
+            x_store(0, x_raw);
+        }
     }
 
     // One step: 64 columns.  The activations of the next step are requested first; the weights are
@@ -492,7 +553,8 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
     constexpr int kChunkValu = C::kNvq ? 72 : C::kMx ? 12 : C::kBits == 3 ? 40 : 32;
     // ... and of the last chunk of a step, which also sets up the next step's lane blocks and requests packed rows
     constexpr int kLastValu = kChunkValu + (C::kNint ? 72 : C::kNvq ? 56 : 20);
-    auto step_piped = [&](int step, FastRaw<CLS> (&raw)[2], const FastRaw<CLS> (&raw_next)[2]) {
+    auto step_piped = [&](int step, FastRaw<CLS> (&raw)[2], FastRaw<CLS> (&raw_next)[2], auto odd_step) {
+        constexpr bool kOdd = decltype(odd_step)::value;
         half8_t aq[MT];
         a_read(step, 0, aq);
         x_direct(step + 1 < steps ? step + 1 : steps - 1);
@@ -510,7 +572,16 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
             } else {
                 // every chunk of this step is decoded: the packed registers take the step after next, and the
                 // first chunk of the next step is decoded from the other ring slot (into wq: b0 and b1 hold this chunk)
-                fetch(step + 2, raw);
+                if constexpr (kStaged) {
+                    if constexpr (kOdd) {
+                        // the runs of the next two steps into both ring slots, the runs of the two after them requested
+                        stage_commit(raw_next, raw);
+                        stage_issue((step + 3) / 2);
+                    }
+                    fetch_scales(step + 2, raw);
+                } else {
+                    fetch(step + 2, raw);
+                }
                 decode_first(step + 1, raw_next);
             }
 #pragma unroll
@@ -546,7 +617,8 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         }
         __builtin_amdgcn_sched_barrier(0);
         // this wave's direct loads have landed; only the weight loads issued after them may be pending
-        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * fetch_loads<CLS>()) : "memory");
+        constexpr int kLoadsBehind = kStaged ? (kOdd ? 4 : 0) + kScaleLoads : 2 * fetch_loads<CLS>();
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kLoadsBehind) : "memory");
         __syncthreads();
     };
     const int run = C::kNvq ? side_run : level_run;
@@ -559,8 +631,8 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         if constexpr (PACKED) {
             decode_first(from, ring[0]);     // `from` is even: the run's first step reads ring slot 0
             for (int step = from; step < to; step += 2) {
-                step_piped(step, ring[0], ring[1]);
-                step_piped(step + 1, ring[1], ring[0]);
+                step_piped(step, ring[0], ring[1], std::false_type{});
+                step_piped(step + 1, ring[1], ring[0], std::true_type{});
             }
         } else {
             for (int step = from; step < to; step += 2) {
