@@ -126,20 +126,21 @@ constexpr int kFastTileN = 256;          // output rows per block: 64 per wave
 constexpr int kFastXRow = 144;           // bytes per LDS row: 64 columns of fp16 and 16 bytes that skew the banks
 constexpr int kFastXBytes = kPrefillTileM * kFastXRow;
 constexpr int kFastLdsBytes = 2 * kFastXBytes;      // activation buffers; the table region and the pair ids follow
-// NINT group levels of the block's rows are staged in LDS for a run of steps at a time (in the place
-// of the NVQ tables): a window of kLevelWindow levels per row and array.  Reading them per step from
-// memory would keep two more cache lines per row alive for the whole block, which the L2 cannot hold.
+// NINT group levels and MXFP4 block scales of the block's rows are staged in LDS for a run of steps at a
+// time (in the place of the NVQ tables): a window of levels per row and array.  Reading them per step from
+// memory would keep more cache lines per row alive for the whole block than the L2 can hold, and a load of
+// one byte per lane touches as many cache lines as the wave has rows.
 constexpr int kOutPitch = 2 * kFastTileN + 16;      // bytes per pair of the output tile staged in LDS
 // NVQ sign masks and group states of the block's rows are staged the same way, behind the NVQ tables:
 // what the tables of the pool leave of their region plus kSideExtraBytes, for runs of up to
 // kSideMaxRun steps.
-constexpr int kSideExtraBytes = 7168;
+constexpr int kSideExtraBytes = 9600;
 constexpr int kTilesFastLdsBytes = kFastLdsBytes + kNvqFastLdsBytes + kSideExtraBytes + kPrefillTileM * 4;   // dynamic LDS of the tile kernel
-constexpr int kSideMaxRun = 8;
-constexpr int kLevelWindow = 64;
-constexpr int kLevelPitch = kLevelWindow + 4;
-static_assert(2 * kFastTileN * kLevelPitch <= kNvqFastLdsBytes, "the level windows share the table region");
+static_assert(kTilesFastLdsBytes == 80 * 1024, "two blocks share the 160 KB of a CU");
 static_assert(kPrefillTileM * kOutPitch <= kFastLdsBytes + kNvqFastLdsBytes, "the output tile reuses the buffers and tables");
+// Tiles of at most 64 pairs (two groups of 32) need 8 KB per activation buffer instead of 18: the table region
+// starts that much earlier and holds longer windows, so that such a tile restages them less often or never.
+constexpr int kLowTileGroups = 2;
 
 __device__ __forceinline__ half8_t as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
     return __builtin_bit_cast(half8_t, u32x4{a, b, c, d});
@@ -156,7 +157,7 @@ template <int CLS> __host__ __device__ constexpr int tile_layout() {
 template <int CLS>
 constexpr int fetch_loads() {
     using C = FastClass<CLS>;
-    return C::kNvq ? 2 : C::kMx ? 2 : C::kQ == 8 ? 2 : 1;
+    return C::kNvq ? 2 : C::kQ == 8 ? 2 : 1;
 }
 
 // Swizzle of the packed activation tile in LDS: rows of 128 bytes, the 16-byte piece c of row r sits at
@@ -170,9 +171,19 @@ template <int CLS, int MT, int IB, bool PACKED>
 __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, int row_block, int pool_index, int local, int begin,
                                                  int count, unsigned char* lds) {
     using C = FastClass<CLS>;
+    // LDS: two activation buffers | the waves' pieces for packed rows (kStaged) | tables and windows | pair ids
+    constexpr bool kLow = PACKED && MT <= kLowTileGroups;
+    constexpr bool kStaged = kLow && (CLS == K_NINT_4_24 || CLS == K_NINT_4_32 || CLS == K_MXFP4);
+    constexpr int kXBytes = kLow ? kLowTileGroups * 32 * 128 : kFastXBytes;      // one activation buffer
+    constexpr int kTablesAt = 2 * kXBytes + (kStaged ? 4 * 4096 : 0);
+    constexpr int kTableRoom = kTilesFastLdsBytes - kPrefillTileM * 4 - kTablesAt;
+    constexpr int kWindow = kLow ? 88 : 64;          // levels per row and array of a window
+    constexpr int kPitch = kWindow + 4;              // an odd number of dwords: the rows of a wave meet no common bank
+    constexpr int kSideMaxRun = kLow ? 16 : 8;       // steps per window of NVQ sign masks and states, at most
+    static_assert(!(C::kNint || C::kMx) || (C::kMx ? 1 : 2) * kFastTileN * kPitch <= kTableRoom, "the level windows fit");
     unsigned char* x_lds = lds;
-    unsigned char* tables = lds + kFastLdsBytes;
-    int* pair_ids = reinterpret_cast<int*>(lds + kFastLdsBytes + kNvqFastLdsBytes + kSideExtraBytes);
+    unsigned char* tables = lds + kTablesAt;
+    int* pair_ids = reinterpret_cast<int*>(lds + kTilesFastLdsBytes - kPrefillTileM * 4);
     const mfq_amd_projection& pool = a.pools[pool_index];
     if (C::kNvq) nvq_fast_tables(pool, tables);
     const FastCtx<CLS> ctx = fast_ctx<CLS>(pool, local, tables);
@@ -207,7 +218,7 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
 #pragma unroll
             for (int k = 0; k < 16; ++k) p[k] = 0u;
         }
-        unsigned char* dst = x_lds + (step & 1) * kFastXBytes + stage_row * kFastXRow + stage_half * 64;
+        unsigned char* dst = x_lds + (step & 1) * kXBytes + stage_row * kFastXRow + stage_half * 64;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             *reinterpret_cast<u32x4*>(dst + 16 * j) = u32x4{p[4 * j], p[4 * j + 1], p[4 * j + 2], p[4 * j + 3]};
@@ -239,7 +250,7 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         const unsigned char* from = reinterpret_cast<const unsigned char*>((static_cast<uintptr_t>(hi) << 32) | lo);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-            unsigned char* to = x_lds + (step & 1) * kFastXBytes + (32 * i + 8 * wave) * 128;
+            unsigned char* to = x_lds + (step & 1) * kXBytes + (32 * i + 8 * wave) * 128;
             // written as assembly so that the compiler does not make every later LDS read wait for it; the
             // waits that cover these loads are the explicit ones before the barriers
             const uint32_t lds_at = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(
@@ -270,27 +281,32 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         int last = steps - 1;
         const LaneBlock b = lane_block<C::kGs>(2 * (step < last ? step : last) + h, width, ctx.groups);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) raw[t] = fast_fetch<CLS, C::kMx>(ctx, b, rows[t]);   // NINT levels, NVQ signs and states come from LDS
+        for (int t = 0; t < 2; ++t) raw[t] = fast_fetch<CLS, false>(ctx, b, rows[t]);   // levels, block scales, signs and states come from LDS
     };
-    // NINT: steps [from, from + run) read their levels from a window of kLevelWindow groups per row
-    const int level_run = C::kNint ? (((kLevelWindow - 2) * C::kGs / 64) & ~1) : steps;
+    // NINT, MXFP4: steps [from, from + run) read their levels from a window of kWindow groups per row.  A lane block
+    // of 32 columns lies in one group of 32 and may straddle two shorter or longer ones.
+    constexpr bool kWindows = C::kNint || C::kMx;
+    constexpr int kWindowArrays = C::kMx ? 1 : 2;
+    const int row_groups = C::kMx ? ctx.row_bytes / 16 : ctx.groups;
+    const int level_run = !kWindows ? steps : C::kGs == 32 ? ((kWindow / 2) & ~1) : (((kWindow - 2) * C::kGs / 64) & ~1);
     int level_first = 0;           // first group of the staged window
     auto stage_levels = [&](int from) {
         level_first = 64 * from / C::kGs;
-        // thread -> one row of the block: up to kLevelWindow bytes of each array, every load issued before
+        // thread -> one row of the block: up to kWindow bytes of each array, every load issued before
         // the first store so that the copy costs one memory round trip
-        const int64_t level_bytes = static_cast<int64_t>(pool.output_rows) * ctx.groups;   // per expert and array
-        const int left = ctx.groups - level_first + 1;
-        const int want = left < kLevelWindow ? left : kLevelWindow;
+        const int64_t level_bytes = static_cast<int64_t>(pool.output_rows) * row_groups;   // per expert and array
+        const int left = row_groups - level_first + 1;
+        const int want = left < kWindow ? left : kWindow;
         int row = row_block * kFastTileN + tid;
         row = row < a.out_rows ? row : a.out_rows - 1;
-        const int64_t at = static_cast<int64_t>(row) * ctx.groups + level_first;
-        u32x4 piece[2][kLevelWindow / 16];
+        const int64_t at = static_cast<int64_t>(row) * row_groups + level_first;
+        constexpr int kPieces = (kWindow + 15) / 16;
+        u32x4 piece[kWindowArrays][kPieces];
 #pragma unroll
-        for (int which = 0; which < 2; ++which) {
+        for (int which = 0; which < kWindowArrays; ++which) {
             const uint8_t* base = which ? ctx.f2 : ctx.f1;
 #pragma unroll
-            for (int q = 0; q < kLevelWindow / 16; ++q) {
+            for (int q = 0; q < kPieces; ++q) {
                 piece[which][q] = u32x4{0u, 0u, 0u, 0u};
                 if (16 * q >= want) continue;
                 if (at + 16 * q + 16 <= level_bytes) {
@@ -304,16 +320,21 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
             }
         }
 #pragma unroll
-        for (int which = 0; which < 2; ++which)
+        for (int which = 0; which < kWindowArrays; ++which)
 #pragma unroll
-            for (int q = 0; q < kLevelWindow / 16; ++q)
+            for (int q = 0; q < kPieces; ++q)
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
-                    *reinterpret_cast<uint32_t*>(tables + (which * kFastTileN + tid) * kLevelPitch + 16 * q + 4 * k) = piece[which][q][k];
+                    if (16 * q + 4 * k < kPitch)
+                        *reinterpret_cast<uint32_t*>(tables + (which * kFastTileN + tid) * kPitch + 16 * q + 4 * k) = piece[which][q][k];
     };
     auto level_pair = [&](int which, int t, const LaneBlock& b) {
-        const unsigned char* at = tables + (which * kFastTileN + wave * 64 + 32 * t + n) * kLevelPitch + (b.group - level_first);
+        const unsigned char* at = tables + (which * kFastTileN + wave * 64 + 32 * t + n) * kPitch + (b.group - level_first);
         return static_cast<uint32_t>(at[0]) | (static_cast<uint32_t>(at[1]) << 8);
+    };
+    // MXFP4: the scale byte of lane block b of row t (a lane block is one group)
+    auto scale_byte = [&](int t, const LaneBlock& b) {
+        return static_cast<uint32_t>(tables[(wave * 64 + 32 * t + n) * kPitch + (b.cb - level_first)]);
     };
 
     // NVQ: steps [from, from + run) read sign masks and states from LDS windows of one row each
@@ -322,14 +343,21 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
     if constexpr (C::kNvq) {
         const int banks = nvq_format_jsc(pool.format) ? static_cast<uint8_t>(static_cast<const int8_t*>(pool.fields[4])[1]) : 1;
         const int used = (64 + 64 + 128 * 16 + banks * ctx.entries * 8 + 15) / 16 * 16;
-        const int room = kNvqFastLdsBytes + kSideExtraBytes - used;
+        const int room = kTableRoom - used;
         side = tables + used;
         // per row and step: 7 bytes of sign masks (two lane blocks of 28 bits) and at most 8/3 states of 4 bits
+        // (a window of an odd number of dwords per row, so that the rows of a wave meet no common bank; no longer
+        // than the row itself)
+        auto pitch_of = [](int w) {
+            const int bytes = ((7 * w + 4 + 3) & ~3) + (((4 * w + 3) / 3 + 4 + 3) & ~3);
+            return (bytes & 4) ? bytes : bytes + 4;
+        };
+        const int longest = steps < kSideMaxRun ? steps : kSideMaxRun;
         side_run = 2;
-        for (int w = 4; w <= kSideMaxRun; w += 2)
-            if (kFastTileN * (((7 * w + 4 + 3) & ~3) + (((4 * w + 3) / 3 + 4 + 3) & ~3)) <= room) side_run = w;
+        for (int w = 4; w <= longest; w += 2)
+            if (kFastTileN * pitch_of(w) <= room) side_run = w;
         side_sign_bytes = (7 * side_run + 4 + 3) & ~3;
-        side_pitch = side_sign_bytes + (((4 * side_run + 3) / 3 + 4 + 3) & ~3);
+        side_pitch = pitch_of(side_run);
     }
     // first byte of the window of row `row` in the sign / state stream for a run that starts at step `from`
     auto sign_start = [&](int row, int from) {
@@ -383,19 +411,16 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         states = state_word >> (state_bit & 7u);
     };
 
-    // Packed rows in coalesced runs (tiles of at most 64 pairs, classes whose lane blocks hold 16 bytes).  A weight load
-    // of the lane that will decode the data touches 32 rows x 32 bytes, and the address unit's time per load instruction
-    // follows the cache lines it touches, not the bytes it brings.  Here a wave loads the 64-byte runs that its 64 rows
-    // need for two steps with four lanes per row (16 rows per instruction: half the lines), parks them in a 4 KB
-    // piece of LDS of its own (the part of the activation buffers that tiles of this height leave unused) and reads them
-    // back in the layout of the MFMA operand, one 16-byte piece per lane, row and step.  Nothing is shared between
-    // waves, so no barrier is involved; the pieces of a row are swizzled so that neither the writes nor the reads meet
-    // in a bank.  The runs of the pair of steps after next are requested when those of the next pair have been read
-    // back, two steps before they are needed.
-    constexpr bool kStaged = PACKED && MT <= 2 && (CLS == K_NINT_4_24 || CLS == K_NINT_4_32 || CLS == K_MXFP4);
-    static_assert(!kStaged || 2 * 32 * 128 + 2 * 4096 <= kFastXBytes, "two waves park their runs behind the rows of a low tile");
+    // Packed rows in coalesced runs (kStaged: tiles of at most 64 pairs, classes whose lane blocks hold 16 bytes).  A
+    // weight load of the lane that will decode the data touches 32 rows x 32 bytes, and the address unit's time per load
+    // instruction follows the cache lines it touches, not the bytes it brings.  Here a wave loads the 64-byte runs that
+    // its 64 rows need for two steps with four lanes per row (16 rows per instruction: half the lines), parks them in a
+    // 4 KB piece of LDS of its own and reads them back in the layout of the MFMA operand, one 16-byte piece per lane,
+    // row and step.  Nothing is shared between waves, so no barrier is involved; the pieces of a row are swizzled so
+    // that neither the writes nor the reads meet in a bank.  The runs of the pair of steps after next are requested when
+    // those of the next pair have been read back, two steps before they are needed.
     u32x4 staged_rows[4] = {};
-    unsigned char* wave_stage = x_lds + (wave >> 1) * kFastXBytes + 2 * 32 * 128 + (wave & 1) * 4096;
+    unsigned char* wave_stage = lds + 2 * kXBytes + wave * 4096;
     auto stage_issue = [&](int pair_of_steps) {
         const int last = steps / 2 - 1;
         const int d = pair_of_steps < last ? pair_of_steps : last;
@@ -424,16 +449,6 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
             for (int k = 0; k < 4; ++k) { even[t].q[k] = first[k]; odd[t].q[k] = second[k]; }
         }
     };
-    // MXFP4: the block scales still come one byte per lane, row and step
-    auto fetch_scales = [&](int step, FastRaw<CLS> (&raw)[2]) {
-        if constexpr (C::kMx) {
-            const int last = steps - 1;
-            const LaneBlock b = lane_block<C::kGs>(2 * (step < last ? step : last) + h, width, ctx.groups);
-#pragma unroll
-            for (int t = 0; t < 2; ++t) raw[t].a = gload<uint8_t>(ctx.f1 + mx_fetch_at(rows[t], ctx.row_bytes, b).scale_byte);
-        }
-    };
-    constexpr int kScaleLoads = C::kMx ? 2 : 0;      // per call of fetch_scales
 
     float16_t acc[2][MT];
 #pragma unroll
@@ -452,9 +467,7 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
     }
     if constexpr (kStaged) {
         stage_issue(0);
-        fetch_scales(0, ring[0]);
-        fetch_scales(1, ring[1]);
-        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(4 + 2 * kScaleLoads) : "memory");   // the direct loads, not the weights
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");   // the direct loads, not the weights
         stage_commit(ring[0], ring[1]);
         stage_issue(1);
     } else {
@@ -482,9 +495,10 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
             uint32_t scales = 0, minima = 0;
             if constexpr (C::kNint) { scales = level_pair(0, t, b); minima = level_pair(1, t, b); }
             if constexpr (C::kNvq) side_pair(t, b, scales, minima);
+            if constexpr (C::kMx) raw[t].a = scale_byte(t, b);
             block[t] = weight_block<CLS>(ctx, b, raw[t], scale[t], scales, minima);
         }
-        const unsigned char* x_tile = x_lds + (step & 1) * kFastXBytes + (PACKED ? 0 : n * kFastXRow + h * 64);
+        const unsigned char* x_tile = x_lds + (step & 1) * kXBytes + (PACKED ? 0 : n * kFastXRow + h * 64);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             uint32_t w[2][4];
@@ -533,11 +547,11 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
     WeightBlock<CLS> block[2];
     uint32_t wq[2][4];
     auto a_read = [&](int step, int j, half8_t (&av)[MT]) {
-        const unsigned char* x_tile = x_lds + (step & 1) * kFastXBytes;
+        const unsigned char* x_tile = x_lds + (step & 1) * kXBytes;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) av[mt] = *reinterpret_cast<const half8_t*>(x_tile + mt * 32 * 128 + a_piece[mt & 1][j]);
     };
-    auto decode_first = [&](int step, const FastRaw<CLS> (&raw)[2]) {
+    auto decode_first = [&](int step, FastRaw<CLS> (&raw)[2]) {
         const int last = steps - 1;
         const LaneBlock b = lane_block<C::kGs>(2 * (step < last ? step : last) + h, width, ctx.groups);
 #pragma unroll
@@ -545,6 +559,7 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
             uint32_t scales = 0, minima = 0;
             if constexpr (C::kNint) { scales = level_pair(0, t, b); minima = level_pair(1, t, b); }
             if constexpr (C::kNvq) side_pair(t, b, scales, minima);
+            if constexpr (C::kMx) raw[t].a = scale_byte(t, b);
             block[t] = weight_block<CLS>(ctx, b, raw[t], scale[t], scales, minima);
             chunk_weights<CLS, IB>(block[t], raw[t], 0, wq[t]);
         }
@@ -578,7 +593,6 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
                         stage_commit(raw_next, raw);
                         stage_issue((step + 3) / 2);
                     }
-                    fetch_scales(step + 2, raw);
                 } else {
                     fetch(step + 2, raw);
                 }
@@ -617,14 +631,14 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         }
         __builtin_amdgcn_sched_barrier(0);
         // this wave's direct loads have landed; only the weight loads issued after them may be pending
-        constexpr int kLoadsBehind = kStaged ? (kOdd ? 4 : 0) + kScaleLoads : 2 * fetch_loads<CLS>();
+        constexpr int kLoadsBehind = kStaged ? (kOdd ? 4 : 0) : 2 * fetch_loads<CLS>();
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kLoadsBehind) : "memory");
         __syncthreads();
     };
     const int run = C::kNvq ? side_run : level_run;
     for (int from = 0; from < steps; from += run) {
         // every wave is past the last step of the previous run (its closing barrier) when the window moves
-        if constexpr (C::kNint) stage_levels(from);
+        if constexpr (kWindows) stage_levels(from);
         if constexpr (C::kNvq) stage_side(from);
         __syncthreads();
         const int to = from + run < steps ? from + run : steps;
