@@ -377,6 +377,33 @@ def test_prefill_uniform_layer(uniform):
     assert err <= FFN_TOL
 
 
+@pytest.mark.parametrize("uniform", ["NINT2", "NINT3", "NINT4", "NVQ3J-L", "MXFP4"])
+def test_prefill_rows_longer_than_a_window(uniform):
+    """4096 and 3072 columns are 64 and 48 steps of the tile kernel: more than one window of group levels (NINT),
+    block scales (MXFP4) or sign masks and states (NVQ) holds, at either tile height, so the windows move inside a
+    block.  Zipf routing over six experts gives tiles of every height: the popular experts fill tiles of 128 pairs,
+    the others stay at or below 64, where the windows are the longer ones."""
+    import torch
+    from mfq_amd import runtime as R
+    import synth
+    experts, inter, k, tokens = 6, 128, 3, 220
+    for hidden in (4096, 3072):
+        # quantised weights where the packer is quick; random codes, sign masks and states for NVQ (its search over the
+        # codebook takes minutes at this width)
+        mode = "random" if uniform.startswith("NVQ") else "pack"
+        tensors, runtimes, _ = _layer(f"test/moe/prefill/long/{uniform}/{hidden}", experts, hidden, inter, mode, uniform=uniform)
+        x = synth.to_bf16(synth.normal(f"test/prefill/long/x/{hidden}", (tokens, hidden)))
+        ids = synth.zipf_routes("test/prefill/long/ids", tokens, experts, k)
+        counts = np.bincount(ids.ravel(), minlength=experts)
+        assert counts.max() > 128 and 0 < counts.min() <= 64, "the case needs tall and low tiles"
+        weights = np.full((tokens, k), 1.0 / k, dtype=np.float32)
+        out = R.MfeFfnRuntime(*runtimes, top_k=k, max_tokens=tokens).run(
+            torch.from_numpy(x).to(torch.bfloat16).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(weights).cuda()).cpu().numpy()
+        err = rel_l2(out, oracle_layer(x, ids, weights, tensors))
+        print(f"prefill {uniform} H={hidden}: pairs per expert {sorted(counts.tolist())} rel-L2 {err:.3e}")
+        assert err <= FFN_TOL
+
+
 def test_prefill_f16_activations_and_stage_buffers():
     """fp16 activations take the pair shuffle without conversion; gate/up and pair outputs match the oracle stages."""
     import torch
