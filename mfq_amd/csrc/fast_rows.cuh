@@ -46,7 +46,60 @@ struct XSource {
     bool vector_ok;
     const float* scale;  // kXScaled: {2^-e, 2^e} of the row, readable once the prologue has run
 };
-constexpr int kXRaw = 0, kXPacked = 1, kXScaled = 2;
+constexpr int kXRaw = 0, kXPacked = 1, kXScaled = 2, kXStaged = 3;
+// kXStaged: the block has packed the token's row into LDS once (stage_x_row): per lane block of 32 columns the 16
+// fp16 pairs in the pair layout of the class and the four chunk sums, kXStagedDwords dwords; XSource::row points
+// there and XSource::scale to the factor that scales results back.  Both are readable once the prologue has run.
+constexpr int kXStagedDwords = 20;
+
+// One token's activation row into LDS in the kXStaged form; every thread of the block calls it (two barriers inside).
+// Thread t packs lane block t, with the arithmetic of pack_block(); `scratch` holds one float per wave.
+template <int CLS>
+__device__ __forceinline__ void stage_x_row(const void* src, int dtype, bool vector_ok, int width, uint32_t* dst, float* up_out,
+                                            float* scratch) {
+    const int lane_blocks = (width + kLaneColumns - 1) / kLaneColumns;
+    const int t = threadIdx.x;
+    const bool active = t < lane_blocks;
+    float values[32];
+    float largest = 0.0f;
+    if (active) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_x8(src, dtype, 4 * t + j, width, vector_ok, &values[8 * j]);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) largest = fmaxf(largest, fabsf(values[i]));
+    }
+    largest = wave_max(largest);
+    if (t % kWave == 0) scratch[t / kWave] = largest;
+    __syncthreads();
+    const int waves = (static_cast<int>(blockDim.x) + kWave - 1) / kWave;
+    for (int w = 0; w < waves; ++w) largest = fmaxf(largest, scratch[w]);
+    float down, up;
+    normaliser(largest, down, up);
+    if (t == 0) *up_out = up;
+    if (active) {
+        _Float16 h[32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) h[i] = static_cast<_Float16>(values[i] * down);
+        uint32_t out[kXStagedDwords];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const int first = pair_column<CLS>(k, 0), second = pair_column<CLS>(k, 1);
+            half2_t pair;
+            pair[0] = static_cast<_Float16>(static_cast<float>(h[first]) * pair_scale<CLS>(k));
+            pair[1] = static_cast<_Float16>(static_cast<float>(h[second]) * pair_scale<CLS>(k));
+            out[k] = __builtin_bit_cast(uint32_t, pair);
+        }
+        float plain[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < 32; ++i) plain[i / 8] += static_cast<float>(h[i]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) out[16 + j] = __float_as_uint(plain[j]);
+#pragma unroll
+        for (int q = 0; q < kXStagedDwords / 4; ++q)
+            *reinterpret_cast<u32x4*>(dst + t * kXStagedDwords + 4 * q) = u32x4{out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]};
+    }
+    __syncthreads();
+}
 struct NoPrologue { __device__ __forceinline__ void operator()() const {} };
 
 // Rows [row_begin, row_end) of one expert times NT tokens.  LPR lanes share a row (64, or 16 when the
@@ -162,6 +215,29 @@ __device__ __forceinline__ void fast_rows(const FastCtx<CLS>& c, const XSource (
             up[n] = gload<float>(row + xpack_scale_at(width));
 #pragma unroll
             for (int s = 0; s < SLABS; ++s) xpack_load<CLS>(row, width, blocks[s], x[s][n]);
+        } else if constexpr (XMODE == kXStaged) {
+            typedef const __attribute__((address_space(3))) u32x4* lds4;
+            up[n] = *xs[n].scale;
+#pragma unroll
+            for (int s = 0; s < SLABS; ++s) {
+                const LaneBlock& b = blocks[s];
+                const lds4 at = (lds4)(static_cast<const uint32_t*>(xs[n].row) + b.cb * kXStagedDwords);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const u32x4 v = at[i];
+                    x[s][n].p[4 * i] = b.valid ? v[0] : 0u; x[s][n].p[4 * i + 1] = b.valid ? v[1] : 0u;
+                    x[s][n].p[4 * i + 2] = b.valid ? v[2] : 0u; x[s][n].p[4 * i + 3] = b.valid ? v[3] : 0u;
+                }
+                const u32x4 plain = at[4];
+                x[s][n].g0 = x[s][n].g1 = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const bool second = (b.sel >> j) & 1u;
+                    const float value = b.valid ? __uint_as_float(plain[j]) : 0.0f;
+                    x[s][n].g0 += second ? 0.0f : value;
+                    x[s][n].g1 += second ? value : 0.0f;
+                }
+            }
         } else {
             float values[SLABS][32];
             float largest = 0.0f;

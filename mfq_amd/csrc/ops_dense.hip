@@ -165,12 +165,27 @@ __global__ void __launch_bounds__(256) gemv_fast_kernel(mfq_amd_projection p, in
                                                         int x_dtype, int batch, int64_t x_stride, float* y,
                                                         int64_t y_stride, int vector_ok) {
     extern __shared__ unsigned char lds[];
-    // the LDS tables of an NVQ pool are built behind the first requests for packed rows (every wave of the block
-    // takes part: there is a barrier inside)
+    // LDS: the tables of an NVQ pool | scale per token, a float per wave | the packed rows of the block's tokens
+    unsigned char* x_area = lds + (FastClass<CLS>::kNvq ? kNvqFastLdsBytes : 0);
+    float* x_up = reinterpret_cast<float*>(x_area);
+    float* x_scratch = x_up + 8;
+    uint32_t* x_rows = reinterpret_cast<uint32_t*>(x_area + 64);
+    const int lane_blocks = (p.input_width + kLaneColumns - 1) / kLaneColumns;
+    const int element = x_dtype == MFQ_AMD_F32 ? 4 : 2;
+    const int first = blockIdx.y * NT;
+    // Behind the first requests for packed rows (every wave of the block takes part: there are barriers inside) the
+    // block builds the LDS tables of an NVQ pool and packs the activation rows of its tokens, once for its four
+    // waves: a wave that packs its own copy spends more instructions on that than on the rows it multiplies.
     auto prologue = [&] {
         if (FastClass<CLS>::kNvq) {
             nvq_fast_tables(p, lds);
             __syncthreads();
+        }
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+            const int token = first + n < batch ? first + n : batch - 1;
+            stage_x_row<CLS>(static_cast<const char*>(x) + static_cast<int64_t>(token) * x_stride * element, x_dtype,
+                             vector_ok != 0, p.input_width, x_rows + n * lane_blocks * kXStagedDwords, x_up + n, x_scratch);
         }
     };
     const FastCtx<CLS> ctx = fast_ctx<CLS>(p, local_expert, lds);
@@ -179,16 +194,11 @@ __global__ void __launch_bounds__(256) gemv_fast_kernel(mfq_amd_projection p, in
     const int row_begin = (blockIdx.x * 4 + wave) * kRowsPerWave;
     if (row_begin >= p.output_rows) { prologue(); return; }
     const int row_end = row_begin + kRowsPerWave < p.output_rows ? row_begin + kRowsPerWave : p.output_rows;
-    const int element = x_dtype == MFQ_AMD_F32 ? 4 : 2;
-    constexpr int kRing = SLABS > 1 ? 4 : (FastClass<CLS>::kRing < SLOTS ? FastClass<CLS>::kRing : SLOTS);
-    const int first = blockIdx.y * NT;
+    constexpr int kRing = SLABS > 1 ? (SLOTS < 4 ? SLOTS : 4) : (FastClass<CLS>::kRing < SLOTS ? FastClass<CLS>::kRing : SLOTS);
     XSource xs[NT];
 #pragma unroll
-    for (int n = 0; n < NT; ++n) {
-        const int token = first + n < batch ? first + n : batch - 1;
-        xs[n] = XSource{static_cast<const char*>(x) + static_cast<int64_t>(token) * x_stride * element, x_dtype, vector_ok != 0, nullptr};
-    }
-    fast_rows<CLS, LPR, SLABS, NT, kRing, kXRaw, SLOTS>(ctx, xs, p.input_width, row_begin, row_end, p.output_rows,
+    for (int n = 0; n < NT; ++n) xs[n] = XSource{x_rows + n * lane_blocks * kXStagedDwords, x_dtype, false, x_up + n};
+    fast_rows<CLS, LPR, SLABS, NT, kRing, kXStaged, SLOTS>(ctx, xs, p.input_width, row_begin, row_end, p.output_rows,
         [&](int n, int row, float value) { if (first + n < batch) y[static_cast<int64_t>(first + n) * y_stride + row] = value; }, prologue);
 }
 
@@ -198,18 +208,19 @@ struct GemvFastLaunch {
     template <int CLS, int LPR, int SLABS, int SLOTS> void go() const {
         constexpr int kRowsPerBlock = 4 * SLOTS * (kWave / LPR);
         const unsigned blocks = (p.output_rows + kRowsPerBlock - 1) / kRowsPerBlock;
-        const int bytes = FastClass<CLS>::kNvq ? kNvqFastLdsBytes : 0;
+        const int lane_blocks = (p.input_width + kLaneColumns - 1) / kLaneColumns;
+        auto lds_bytes = [&](int tokens) { return (FastClass<CLS>::kNvq ? kNvqFastLdsBytes : 0) + 64 + tokens * lane_blocks * kXStagedDwords * 4; };
         // Two tokens per block where decoding a row costs more than reading it again: NVQ rows of two slabs
         // (measured at 4096 x 4096: batch 16 in 38 us instead of 57 us; the other classes lose parallelism
         // and run slower in groups).
         if constexpr (FastClass<CLS>::kNvq && SLABS > 1) {
             if (batch >= 2) {
-                hipLaunchKernelGGL((gemv_fast_kernel<CLS, LPR, SLABS, SLOTS, 2>), dim3(blocks, (batch + 1) / 2), dim3(256), bytes,
+                hipLaunchKernelGGL((gemv_fast_kernel<CLS, LPR, SLABS, SLOTS, 2>), dim3(blocks, (batch + 1) / 2), dim3(256), lds_bytes(2),
                                    stream, p, local_expert, x, x_dtype, batch, x_stride, y, y_stride, vector_ok);
                 return;
             }
         }
-        hipLaunchKernelGGL((gemv_fast_kernel<CLS, LPR, SLABS, SLOTS, 1>), dim3(blocks, batch), dim3(256), bytes, stream, p,
+        hipLaunchKernelGGL((gemv_fast_kernel<CLS, LPR, SLABS, SLOTS, 1>), dim3(blocks, batch), dim3(256), lds_bytes(1), stream, p,
                            local_expert, x, x_dtype, batch, x_stride, y, y_stride, vector_ok);
     }
     template <int CLS> void run() const {
@@ -221,7 +232,14 @@ struct GemvFastLaunch {
             const bool tall = static_cast<int64_t>(p.output_rows) * ((batch + group - 1) / group) >= enough;
             if (p.input_width <= 16 * kLaneColumns) { if (tall) go<CLS, 16, 1, 8>(); else go<CLS, 16, 1, 4>(); }
             else if (p.input_width <= kWave * kLaneColumns) { if (tall) go<CLS, 64, 1, 16>(); else go<CLS, 64, 1, 4>(); }
-            else { if (tall) go<CLS, 64, 2, 8>(); else go<CLS, 64, 2, 4>(); }
+            else {
+                // (NVQ, 4096 x 4096, one token group: 8.5 us with 2 rows per wave, 9.2 us with 4; two groups: 19.2 / 14.2;
+                // NINT4: 6.7 / 6.2 us.  Four tokens per block instead of two: batch 8 in 20.9 us against 20.3.)
+                const bool one_group = (batch + group - 1) / group == 1;
+                if (tall) go<CLS, 64, 2, 8>();
+                else if (FastClass<CLS>::kNvq && one_group) go<CLS, 64, 2, 2>();
+                else go<CLS, 64, 2, 4>();
+            }
         }
     }
 };
