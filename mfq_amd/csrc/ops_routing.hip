@@ -851,7 +851,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_small_kernel(PlanArgs
         expert_of[tid] = -1;
         __syncthreads();
         // a whole wave per token while the block has waves to spare, half a wave beyond that
-        if (a.route.tokens <= kPlanThreads / 128) {
+        if (a.route.tokens <= kPlanThreads / 64) {
             const int token = tid >> 6;
             topk_token<(TOPK_SLOTS >= 2 ? TOPK_SLOTS / 2 : 1), 64>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
                                                                    a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
@@ -1078,7 +1078,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_pairs_kernel(PlanArgs
     for (int s = 0; s < kSlots; ++s) words[s] = s < x.slots && tid < E ? x.expert_words[s * E + tid] : kExpertAbsent;
     if (TOPK_SLOTS > 0) {
         // a whole wave per token while the block has waves to spare, half a wave beyond that
-        if (a.route.tokens <= kPlanThreads / 128) {
+        if (a.route.tokens <= kPlanThreads / 64) {
             const int token = tid >> 6;
             topk_token<(TOPK_SLOTS >= 2 ? TOPK_SLOTS / 2 : 1), 64>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
                                                                    a.route.normalize, a.route.norm_floor, a.route.scale, a.route.ids_out,
