@@ -850,7 +850,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_small_kernel(PlanArgs
     if (TOPK_SLOTS > 0) {
         expert_of[tid] = -1;
         __syncthreads();
-        // a whole wave per token while the block has waves to spare, half a wave beyond that
+        // a whole wave per token while the block has a wave for each (sixteen), half a wave beyond that
         if (a.route.tokens <= kPlanThreads / 64) {
             const int token = tid >> 6;
             topk_token<(TOPK_SLOTS >= 2 ? TOPK_SLOTS / 2 : 1), 64>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
@@ -1077,7 +1077,7 @@ __global__ void __launch_bounds__(kPlanThreads) route_plan_pairs_kernel(PlanArgs
 #pragma unroll
     for (int s = 0; s < kSlots; ++s) words[s] = s < x.slots && tid < E ? x.expert_words[s * E + tid] : kExpertAbsent;
     if (TOPK_SLOTS > 0) {
-        // a whole wave per token while the block has waves to spare, half a wave beyond that
+        // a whole wave per token while the block has a wave for each (sixteen), half a wave beyond that
         if (a.route.tokens <= kPlanThreads / 64) {
             const int token = tid >> 6;
             topk_token<(TOPK_SLOTS >= 2 ? TOPK_SLOTS / 2 : 1), 64>(a.route.logits, a.route.dtype, token, token < a.route.tokens, E, a.top_k,
