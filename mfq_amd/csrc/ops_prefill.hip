@@ -20,6 +20,7 @@
 #include "launch.cuh"
 #include "moe_args.h"
 #include "tile_pack.cuh"
+#include "tile_windows.h"
 #include "xpack.cuh"
 
 namespace mfq_amd {
@@ -288,15 +289,14 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
     constexpr bool kWindows = C::kNint || C::kMx;
     constexpr int kWindowArrays = C::kMx ? 1 : 2;
     const int row_groups = C::kMx ? ctx.row_bytes / 16 : ctx.groups;
-    const int level_run = !kWindows ? steps : C::kGs == 32 ? ((kWindow / 2) & ~1) : (((kWindow - 2) * C::kGs / 64) & ~1);
+    const int level_run = kWindows ? level_window_run(C::kGs, kWindow) : steps;
     int level_first = 0;           // first group of the staged window
     auto stage_levels = [&](int from) {
-        level_first = 64 * from / C::kGs;
+        level_first = level_window_first(C::kGs, from);
         // thread -> one row of the block: up to kWindow bytes of each array, every load issued before
         // the first store so that the copy costs one memory round trip
         const int64_t level_bytes = static_cast<int64_t>(pool.output_rows) * row_groups;   // per expert and array
-        const int left = row_groups - level_first + 1;
-        const int want = left < kWindow ? left : kWindow;
+        const int want = level_window_bytes(row_groups, level_first, kWindow);
         int row = row_block * kFastTileN + tid;
         row = row < a.out_rows ? row : a.out_rows - 1;
         const int64_t at = static_cast<int64_t>(row) * row_groups + level_first;
@@ -329,12 +329,15 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
                         *reinterpret_cast<uint32_t*>(tables + (which * kFastTileN + tid) * kPitch + 16 * q + 4 * k) = piece[which][q][k];
     };
     auto level_pair = [&](int which, int t, const LaneBlock& b) {
-        const unsigned char* at = tables + (which * kFastTileN + wave * 64 + 32 * t + n) * kPitch + (b.group - level_first);
+        // (a lane block behind the end of the row, which only the converting path meets, multiplies zero activations; it
+        // reads the window's first levels, which are there)
+        const unsigned char* at = tables + (which * kFastTileN + wave * 64 + 32 * t + n) * kPitch + (PACKED || b.valid ? b.group - level_first : 0);
         return static_cast<uint32_t>(at[0]) | (static_cast<uint32_t>(at[1]) << 8);
     };
     // MXFP4: the scale byte of lane block b of row t (a lane block is one group)
     auto scale_byte = [&](int t, const LaneBlock& b) {
-        return static_cast<uint32_t>(tables[(wave * 64 + 32 * t + n) * kPitch + (b.cb - level_first)]);
+        // (behind the end of the row: the window's first scale, a finite factor for weights that meet zero activations)
+        return static_cast<uint32_t>(tables[(wave * 64 + 32 * t + n) * kPitch + (PACKED || b.valid ? b.cb - level_first : 0)]);
     };
 
     // NVQ: steps [from, from + run) read sign masks and states from LDS windows of one row each
@@ -346,26 +349,13 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
         const int room = kTableRoom - used;
         side = tables + used;
         // per row and step: 7 bytes of sign masks (two lane blocks of 28 bits) and at most 8/3 states of 4 bits
-        // (a window of an odd number of dwords per row, so that the rows of a wave meet no common bank; no longer
-        // than the row itself)
-        auto pitch_of = [](int w) {
-            const int bytes = ((7 * w + 4 + 3) & ~3) + (((4 * w + 3) / 3 + 4 + 3) & ~3);
-            return (bytes & 4) ? bytes : bytes + 4;
-        };
-        const int longest = steps < kSideMaxRun ? steps : kSideMaxRun;
-        side_run = 2;
-        for (int w = 4; w <= longest; w += 2)
-            if (kFastTileN * pitch_of(w) <= room) side_run = w;
-        side_sign_bytes = (7 * side_run + 4 + 3) & ~3;
-        side_pitch = pitch_of(side_run);
+        side_run = side_window_run(room, kFastTileN, steps, kSideMaxRun);
+        side_sign_bytes = side_window_sign_bytes(side_run);
+        side_pitch = side_window_pitch(side_run);
     }
     // first byte of the window of row `row` in the sign / state stream for a run that starts at step `from`
-    auto sign_start = [&](int row, int from) {
-        return ((static_cast<uint32_t>(row) * ctx.nsign4 + 2u * from) * 28u + ctx.sign_bit0) >> 3;
-    };
-    auto state_start = [&](int row, int from) {
-        return ((static_cast<uint32_t>(row) * ctx.groups + 64u * from / 24u) * 4u + ctx.state_bit0) >> 3;
-    };
+    auto sign_start = [&](int row, int from) { return side_window_sign_start(row, ctx.nsign4, ctx.sign_bit0, from); };
+    auto state_start = [&](int row, int from) { return side_window_state_start(row, ctx.groups, ctx.state_bit0, from); };
     auto stage_side = [&](int from) {
         side_from = from;
         int row = row_block * kFastTileN + tid;
@@ -402,11 +392,13 @@ __device__ __forceinline__ void tiles_fast_block(const RowsArgs& a, int slot, in
     // sign masks (28 bits from bit 0) and states (8 bits from bit 0) of lane block b of row t
     auto side_pair = [&](int t, const LaneBlock& b, uint32_t& masks, uint32_t& states) {
         const unsigned char* window = side + (wave * 64 + 32 * t + n) * side_pitch;
-        const uint32_t sign_bit = (static_cast<uint32_t>(rows[t]) * ctx.nsign4 + b.cb) * 28u + ctx.sign_bit0;
-        const uint32_t state_bit = (static_cast<uint32_t>(rows[t]) * ctx.groups + b.group) * 4u + ctx.state_bit0;
-        const uint32_t sign_word = *reinterpret_cast<const unaligned_u32*>(window + ((sign_bit >> 3) - sign_start(rows[t], side_from)));
-        const uint32_t state_word = *reinterpret_cast<const unaligned_u16*>(
-            window + side_sign_bytes + ((state_bit >> 3) - state_start(rows[t], side_from)));
+        const uint32_t sign_bit = side_sign_bit(rows[t], ctx.nsign4, ctx.sign_bit0, b.cb);
+        const uint32_t state_bit = side_state_bit(rows[t], ctx.groups, ctx.state_bit0, b.group);
+        // (behind the end of the row: the window's first bytes)
+        const uint32_t sign_at = PACKED || b.valid ? (sign_bit >> 3) - sign_start(rows[t], side_from) : 0u;
+        const uint32_t state_at = PACKED || b.valid ? (state_bit >> 3) - state_start(rows[t], side_from) : 0u;
+        const uint32_t sign_word = *reinterpret_cast<const unaligned_u32*>(window + sign_at);
+        const uint32_t state_word = *reinterpret_cast<const unaligned_u16*>(window + side_sign_bytes + state_at);
         masks = sign_word >> (sign_bit & 7u);
         states = state_word >> (state_bit & 7u);
     };

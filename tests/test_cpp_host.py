@@ -113,6 +113,23 @@ def test_streaming_fetches_stay_inside_their_fields(tmp_path):
     assert "fetches inside their fields" in done.stdout and int(done.stdout.split()[0]) > 1_000_000
 
 
+def test_tile_kernel_windows_hold_what_the_steps_read(tmp_path):
+    """The LDS windows of the prefill tile kernel (mfq_amd/csrc/tile_windows.h), compiled for the host and swept over
+    widths from 64 to 8192, both window lengths, every group size and side windows of up to 8 and 16 steps: every level,
+    block scale, sign mask and state a step reads lies in what its window staged, and the decode one step ahead stays
+    inside the row's own piece of LDS."""
+    import shutil
+    import subprocess
+    compiler = shutil.which("g++") or shutil.which("hipcc")
+    if compiler is None:
+        pytest.skip("no host C++ compiler")
+    binary = tmp_path / "tile_window_check"
+    subprocess.run([compiler, "-O2", "-std=c++17", str(ROOT / "tests" / "cpp" / "tile_window_check.cpp"), "-o", str(binary)], check=True)
+    done = subprocess.run([str(binary)], capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
+    assert "window reads inside what was staged" in done.stdout and int(done.stdout.split()[0]) > 10_000_000
+
+
 def test_e4m3_split_rounding_and_scales(tmp_path):
     """mfq_amd/csrc/fp8_split.h compiled for the host: E4M3 rounding against all byte values (nearest, ties to even,
     saturation), the E8M0 block scale rule, and hi + lo adding up to bf16 sources."""

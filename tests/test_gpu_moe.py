@@ -382,12 +382,13 @@ def test_prefill_rows_longer_than_a_window(uniform):
     """4096 and 3072 columns are 64 and 48 steps of the tile kernel: more than one window of group levels (NINT),
     block scales (MXFP4) or sign masks and states (NVQ) holds, at either tile height, so the windows move inside a
     block.  Zipf routing over six experts gives tiles of every height: the popular experts fill tiles of 128 pairs,
-    the others stay at or below 64, where the windows are the longer ones."""
+    the others stay at or below 64, where the windows are the longer ones.  2144 columns (67 lane blocks) take the
+    converting path, whose last step lies in a second window and ends in a lane block behind the end of the row."""
     import torch
     from mfq_amd import runtime as R
     import synth
     experts, inter, k, tokens = 6, 128, 3, 220
-    for hidden in (4096, 3072):
+    for hidden in (4096, 3072, 2144):
         # quantised weights where the packer is quick; random codes, sign masks and states for NVQ (its search over the
         # codebook takes minutes at this width)
         mode = "random" if uniform.startswith("NVQ") else "pack"
