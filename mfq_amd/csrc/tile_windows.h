@@ -10,10 +10,12 @@ namespace mfq_amd {
 namespace dev {
 
 // ---- NINT group levels, MXFP4 block scales: `window` bytes per row and array, one byte per group ----
-// Steps of one window.  A lane block of 32 columns lies in one group of 32 and may straddle two shorter or longer
-// ones; it reads the level of its first group and of the next.
+// Steps of one window.  A lane block of 32 columns lies in one group of 32 or in two of 16 and may straddle two of
+// another size; it reads the level of its first group and of the next.  Where a step is a whole number of groups
+// (16, 32) a window starts on a step's first group and serves window * group_size / 64 steps; elsewhere the window's
+// first group may begin before the step does and the last block may reach one group further: two levels of slack.
 MFQ_HD constexpr int level_window_run(int group_size, int window) {
-    return group_size == 32 ? ((window / 2) & ~1) : (((window - 2) * group_size / 64) & ~1);
+    return 64 % group_size == 0 ? ((window * group_size / 64) & ~1) : (((window - 2) * group_size / 64) & ~1);
 }
 // First group of the window that serves steps [from, from + run).
 MFQ_HD constexpr int level_window_first(int group_size, int from) { return 64 * from / group_size; }
